@@ -256,8 +256,12 @@ class EmulatedKernels:
 
     def band_norm(self, bands, eps):
         self._count("band_norm")
-        for src, weight, count, out in bands:
+        for band in bands:
+            src, weight, count, out = band[:4]
+            bias = band[4] if len(band) > 4 else None
             v = src.to(self.acc)
+            if bias is not None:
+                v = v + bias.to(self.acc)
             y = v * torch.rsqrt(v.pow(2).sum(-1, keepdim=True) / count + eps) * weight.to(self.acc)
             cols = src.shape[1]
             result = torch.zeros(out.shape, dtype=out.dtype, device=out.device)
@@ -328,9 +332,146 @@ class EmulatedKernels:
         v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
         out.copy_((v.reshape(n, w) * weight.to(self.acc)).to(out.dtype))
 
-    def copy_columns(self, src, out):
+    def copy_columns(self, src, out, scale=1.0):
         self._count("copy_columns")
-        out.copy_(src)
+        out.copy_(src if scale == 1.0 else (src.to(self.acc) * scale).to(out.dtype))
+
+    # ---- a matrix memory a head -------------------------------------------------------------------
+    def memory_inputs(self, row, positions, inv_freq, qk, heads, head_dim, q_scale, k_scale):
+        self._count("memory_inputs")
+        n, width = row.shape[0], heads * head_dim
+        v = row[:, :2 * width].to(self.acc).reshape(n, 2 * heads, head_dim).clone()
+        if inv_freq is not None:
+            half = inv_freq.shape[0]
+            ang = positions.to(torch.float32)[:, None] * inv_freq[None, :]          # float32 angles
+            cos, sin = ang.cos().to(self.acc)[:, None, :], ang.sin().to(self.acc)[:, None, :]
+            a, b = v[..., :half].clone(), v[..., half:2 * half].clone()
+            v[..., :half] = a * cos - b * sin
+            v[..., half:2 * half] = b * cos + a * sin
+        v = v.reshape(n, 2, width)
+        qk[0].copy_((v[:, 0] * q_scale).to(torch.float32))
+        qk[1].copy_((v[:, 1] * k_scale).to(torch.float32))
+
+    def memory_gates(self, gates, i_bias, f_bias, qk, state, carried_offset, seg_q_start, seg_q_len, state_slots, steps,
+                     heads, head_dim, cap, den_eps):
+        self._count("memory_gates")
+        acc = self.acc
+        z = gates.to(acc)
+        zi, zf = z[:, :heads], z[:, heads:2 * heads]
+        if i_bias is not None:
+            zi = zi + i_bias.to(acc)
+        if f_bias is not None:
+            zf = zf + f_bias.to(acc)
+        if cap:
+            zi, zf = cap * torch.tanh(zi / cap), cap * torch.tanh(zf / cap)
+        log_i, log_f = zi, torch.nn.functional.logsigmoid(zf)
+        width = heads * head_dim
+        for seg in range(seg_q_start.shape[0]):
+            start, length, slot = int(seg_q_start[seg]), int(seg_q_len[seg]), int(state_slots[seg])
+            carried = state[slot, carried_offset:carried_offset + width + heads]
+            nv, m = carried[:width].to(acc).view(heads, head_dim).clone(), carried[width:].to(acc).clone()
+            for t in range(start, start + length):
+                m_new = torch.maximum(log_f[t] + m, log_i[t])
+                a, b = torch.exp(log_f[t] + m - m_new), torch.exp(log_i[t] - m_new)
+                q, k = qk[0, t].to(acc).view(heads, head_dim), qk[1, t].to(acc).view(heads, head_dim)
+                nv = a[:, None] * nv + b[:, None] * k
+                m = m_new
+                den = torch.maximum((nv * q).sum(-1).abs(), torch.exp(-m)) + den_eps
+                steps[0, t], steps[1, t], steps[2, t] = a.float(), b.float(), den.float()
+            carried[:width] = nv.reshape(-1).float()
+            carried[width:] = m.float()
+
+    def memory_scan(self, qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads, head_dim, value_dim):
+        self._count("memory_scan")
+        acc = self.acc
+        size = heads * head_dim * value_dim
+        for seg in range(seg_q_start.shape[0]):
+            start, length, slot = int(seg_q_start[seg]), int(seg_q_len[seg]), int(state_slots[seg])
+            S = state[slot, :size].to(acc).view(heads, head_dim, value_dim).clone()
+            for t in range(start, start + length):
+                q, k = qk[0, t].to(acc).view(heads, head_dim), qk[1, t].to(acc).view(heads, head_dim)
+                val = v[t].to(acc).view(heads, value_dim)
+                if steps is not None:
+                    a, b, den = steps[0, t].to(acc), steps[1, t].to(acc), steps[2, t].to(acc)
+                else:
+                    a, b, den = decays.to(acc), torch.ones(heads, dtype=acc), torch.ones(heads, dtype=acc)
+                S = a[:, None, None] * S + (b[:, None] * k)[:, :, None] * val[:, None, :]
+                y[t] = (torch.einsum("hdv,hd->hv", S, q) / den[:, None]).reshape(-1).float()
+            state[slot, :size] = S.reshape(-1).float()
+
+    def head_norm_gate(self, y, gate, weight, out, heads, eps, activation, scale):
+        self._count("head_norm_gate")
+        n, w = y.shape
+        v = y.to(self.acc).view(n, heads, w // heads)
+        v = (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(n, w)
+        if weight is not None:
+            v = v * weight.to(self.acc)
+        z = gate.to(self.acc)
+        act = torch.sigmoid(z) if activation == "sigmoid" else z * torch.sigmoid(z)
+        out.copy_((v * act * scale).to(out.dtype))
+
+    # ---- a mixture of experts ---------------------------------------------------------------------
+    def moe_route(self, x, router, ids, weights, groups, keep, eps):
+        self._count("moe_route")
+        n, experts, top = x.shape[0], router.shape[0], ids.shape[1]
+        s = torch.softmax(x.to(self.acc) @ router.to(self.acc).T, dim=-1)
+        allowed = torch.ones(n, experts, dtype=torch.bool)
+        if keep < groups:
+            per = experts // groups
+            best = s.view(n, groups, per).max(-1).values
+            kept = torch.zeros(n, groups, dtype=torch.bool)
+            for r in range(n):
+                order = sorted(range(groups), key=lambda g: (-float(best[r, g]), g))
+                kept[r, order[:keep]] = True
+            allowed = kept[:, :, None].expand(n, groups, per).reshape(n, experts)
+        for r in range(n):
+            order = sorted([e for e in range(experts) if allowed[r, e]], key=lambda e: (-float(s[r, e]), e))[:top]
+            chosen = s[r, order]
+            ids[r] = torch.tensor(order, dtype=torch.int32)
+            weights[r] = (chosen / (chosen.sum() + eps)).float()
+
+    def moe_plan(self, ids, plan, experts):
+        self._count("moe_plan")
+        flat = ids.reshape(-1).tolist()
+        max_tiles = len(flat) // 16 + experts
+        plan.fill_(-7)                       # what the kernels must not read
+        tiles = 0
+        for e in range(experts):
+            mine = [a for a, x in enumerate(flat) if x == e]
+            for t0 in range(0, len(mine), 16):
+                rows = mine[t0:t0 + 16]
+                plan[1 + tiles] = e
+                at = 1 + max_tiles + 16 * tiles
+                plan[at:at + 16] = torch.tensor(rows + [-1] * (16 - len(rows)), dtype=torch.int32)
+                tiles += 1
+        plan[0] = tiles
+
+    def _plan_rows(self, plan, experts, assignments):
+        max_tiles = assignments // 16 + experts
+        for t in range(int(plan[0])):
+            at = 1 + max_tiles + 16 * t
+            yield int(plan[1 + t]), [a for a in plan[at:at + 16].tolist() if a >= 0]
+
+    def moe_experts_up(self, x, w, plan, act, top, activation):
+        self._count("moe_experts_up")
+        ff = w.shape[1] // 2
+        for e, rows in self._plan_rows(plan, w.shape[0], act.shape[0]):
+            h = x[[a // top for a in rows]].to(self.acc)
+            z, u = h @ w[e, :ff].to(self.acc).T, h @ w[e, ff:].to(self.acc).T
+            if activation == "gelu_tanh":
+                z = 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+            else:
+                z = z * torch.sigmoid(z)
+            act[rows] = (z * u).to(act.dtype)
+
+    def moe_experts_down(self, act, w, plan, weights, out):
+        self._count("moe_experts_down")
+        n, top = weights.shape
+        flat = weights.reshape(-1)
+        for e, rows in self._plan_rows(plan, w.shape[0], act.shape[0]):
+            y = act[rows].to(self.acc) @ w[e].to(self.acc).T
+            for a, r in zip(rows, y):
+                out[a % top, a // top] = (r * flat[a].to(self.acc)).float()
 
     def stream_add(self, x, addend, delta, delta_bias):
         self._count("stream_add")

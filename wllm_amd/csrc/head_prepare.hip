@@ -294,27 +294,33 @@ WLLM_API int wllm_sigmoid_gate(const void* a, long long a_stride, const void* ga
     return launch_status();
 }
 
-// ---- out[r, c] = src[r, c] with row strides: a tensor into a band of columns of a wider one ------
+// ---- out[r, c] = src[r, c] * scale with row strides: a tensor into a band of columns of a wider one
+// (scale 1: the same bits) ------
 template <typename T>
 __global__ void copy_columns_kernel(const T* __restrict__ src, long long src_stride, T* __restrict__ out,
-                                    long long out_stride, int rows, int cols) {
+                                    long long out_stride, int rows, int cols, float scale) {
     for (int r = blockIdx.y; r < rows; r += gridDim.y) {
         const T* s = src + r * src_stride;
         T* o = out + r * out_stride;
-        for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < cols; c += gridDim.x * blockDim.x) o[c] = s[c];
+        if (scale == 1.f) {
+            for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < cols; c += gridDim.x * blockDim.x) o[c] = s[c];
+        } else {
+            for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < cols; c += gridDim.x * blockDim.x)
+                o[c] = from_float<T>(to_float(s[c]) * scale);
+        }
     }
 }
 
 WLLM_API int wllm_copy_columns(const void* src, long long src_stride, void* out, long long out_stride, int is_bf16,
-                               int rows, int cols, hipStream_t stream) {
+                               int rows, int cols, float scale, hipStream_t stream) {
     if (rows <= 0 || cols <= 0) return 0;
     const dim3 grid(cols < 4096 ? (cols + 255) / 256 : 16, rows < 16384 ? rows : 16384);
     if (is_bf16)
         copy_columns_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(src), src_stride, static_cast<bf16*>(out),
-                                                            out_stride, rows, cols);
+                                                            out_stride, rows, cols, scale);
     else
         copy_columns_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(src), src_stride,
-                                                             static_cast<float*>(out), out_stride, rows, cols);
+                                                             static_cast<float*>(out), out_stride, rows, cols, scale);
     return launch_status();
 }
 

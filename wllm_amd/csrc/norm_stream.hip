@@ -110,8 +110,9 @@ WLLM_API int wllm_norm_add(float* x, const void* delta, int delta_type, int spli
     return launch_status();
 }
 
-// ---- RMS norm of a band of columns of every row, with a weight: out = v / sqrt(sum(v^2) / count + eps) * w.
-// The band [rows, cols] lies in a wider tensor (row stride); `count` is the number of elements the
+// ---- RMS norm of a band of columns of every row, with a weight: out = v / sqrt(sum(v^2) / count + eps) * w,
+// where v is the band, plus a bias (float32, one a column) if the band has one: a projection's bias that
+// belongs in front of its norm.  The band [rows, cols] lies in a wider tensor (row stride); `count` is the number of elements the
 // mean is taken over (less than cols where a band carries padding that is always zero); out may be
 // the band itself or another band, and where it is wider than cols the further columns become zero.
 // Up to two bands a launch (blockIdx.y), each with its own operands. ----
@@ -124,6 +125,7 @@ struct NormBand {
     void* out;
     long long out_stride;
     int out_cols;
+    const float* bias;
 };
 
 template <typename T>
@@ -134,23 +136,24 @@ __global__ void __launch_bounds__(256) band_norm_kernel(NormBand b0, NormBand b1
     T* o = static_cast<T*>(b.out) + static_cast<size_t>(blockIdx.x) * b.out_stride;
     float ss = 0.f;
     for (int i = threadIdx.x; i < b.cols; i += blockDim.x) {
-        const float v = to_float(s[i]);
+        const float v = to_float(s[i]) + (b.bias ? b.bias[i] : 0.f);
         ss += v * v;
     }
     const float inv = 1.f / sqrtf(block_sum(ss, scratch) / b.count + eps);
     for (int i = threadIdx.x; i < b.out_cols; i += blockDim.x)
-        o[i] = from_float<T>(i < b.cols ? to_float(s[i]) * inv * b.weight[i] : 0.f);
+        o[i] = from_float<T>(i < b.cols ? (to_float(s[i]) + (b.bias ? b.bias[i] : 0.f)) * inv * b.weight[i] : 0.f);
 }
 
 WLLM_API int wllm_band_norm(const void* src0, long long src_stride0, int cols0, const float* weight0, float count0,
-                            void* out0, long long out_stride0, int out_cols0, const void* src1, long long src_stride1,
-                            int cols1, const float* weight1, float count1, void* out1, long long out_stride1,
-                            int out_cols1, float eps, int is_bf16, int rows, hipStream_t stream) {
+                            void* out0, long long out_stride0, int out_cols0, const float* bias0, const void* src1,
+                            long long src_stride1, int cols1, const float* weight1, float count1, void* out1,
+                            long long out_stride1, int out_cols1, const float* bias1, float eps, int is_bf16, int rows,
+                            hipStream_t stream) {
     if (rows <= 0) return 0;
     if (!src0 || !out0 || !weight0 || cols0 <= 0 || out_cols0 < cols0 || !(count0 > 0.f)) return -1;
     if (src1 && (!out1 || !weight1 || cols1 <= 0 || out_cols1 < cols1 || !(count1 > 0.f))) return -1;
-    const NormBand b0{src0, src_stride0, cols0, weight0, count0, out0, out_stride0, out_cols0};
-    const NormBand b1{src1, src_stride1, cols1, weight1, count1, out1, out_stride1, out_cols1};
+    const NormBand b0{src0, src_stride0, cols0, weight0, count0, out0, out_stride0, out_cols0, bias0};
+    const NormBand b1{src1, src_stride1, cols1, weight1, count1, out1, out_stride1, out_cols1, bias1};
     const dim3 grid(rows, src1 ? 2 : 1);
     if (is_bf16) band_norm_kernel<bf16><<<grid, 256, 0, stream>>>(b0, b1, eps);
     else band_norm_kernel<float><<<grid, 256, 0, stream>>>(b0, b1, eps);

@@ -432,14 +432,18 @@ def sigmoid_gate(a: torch.Tensor, gate: torch.Tensor, out: torch.Tensor, per: in
             call("sigmoid_gate", a, gate, out)
 
 
-def copy_columns(src: torch.Tensor, out: torch.Tensor) -> None:
-    """out = src; both T [n, c], each possibly a band of columns of a wider tensor."""
+def copy_columns(src: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out = src * scale (in float32, cast to T; scale 1: the same bits); both T [n, c], each possibly a
+    band of columns of a wider tensor; out may be src."""
     _need(src.dim() == 2 and src.dtype in _ACT, "src: expected T [n, c]")
     n, c = src.shape
     _band(src, "src", src.dtype, n, c)
     _band(out, "out", src.dtype, n, c)
     if n and c:
-        call("copy_columns", src, out)
+        if scale != 1.0:
+            call("copy_columns", src, out, float(scale))
+        else:
+            call("copy_columns", src, out)
 
 
 def stream_add(x: torch.Tensor, addend: Optional[torch.Tensor] = None, delta: Optional[torch.Tensor] = None,
@@ -746,15 +750,19 @@ def norm_add(x: torch.Tensor, *, delta: Optional[torch.Tensor] = None, delta_nor
 
 
 def band_norm(bands: list, eps: float) -> None:
-    """RMS norm with a weight over bands of columns: for each (src, weight, count, out) of `bands` (one
-    or two), out[r] = src[r] / sqrt(sum(src[r]^2) / count + eps) * weight.  src T [n, c] and out T
+    """RMS norm with a weight over bands of columns: for each (src, weight, count, out[, bias]) of `bands`
+    (one or two), out[r] = v / sqrt(sum(v^2) / count + eps) * weight with v = src[r] (+ bias, float32 [c]
+    or None: a projection's bias that belongs in front of its norm).  src T [n, c] and out T
     [n, c'] with c' >= c may be bands of wider tensors and may be the same band; columns of out beyond c
     become zero.  weight float32 [c].  `count` is the number of elements the mean is taken over (less
     than c where the band carries padding that is always zero)."""
     _need(1 <= len(bands) <= 2, "bands: one or two")
     n, dtype = bands[0][0].shape[0], bands[0][0].dtype
     _need(dtype in _ACT, "src: expected T")
-    for src, weight, count, out in bands:
+    bands = [tuple(b) + (None,) * (5 - len(b)) for b in bands]
+    for src, weight, count, out, bias in bands:
+        if bias is not None:
+            _dense(bias, "bias", torch.float32, (src.shape[1],))
         _need(src.dim() == 2 and out.dim() == 2 and out.shape[1] >= src.shape[1], "out: at least as wide as src")
         _band(src, "src", dtype, n, src.shape[1])
         _band(out, "out", dtype, n, out.shape[1])
@@ -878,6 +886,204 @@ def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, out
         call("gated_group_norm", y, z, weight, out, int(groups), float(eps))
 
 
+# ---- a matrix memory a head (linear attention in its recurrent form) ------------------------------------
+GATE_KINDS = {"sigmoid": 0, "silu": 1}
+
+
+def _segments(seg_q_start, seg_q_len, state_slots) -> int:
+    s = seg_q_start.shape[0]
+    for t, name in ((seg_q_start, "seg_q_start"), (seg_q_len, "seg_q_len"), (state_slots, "state_slots")):
+        _dense(t, name, torch.int32, (s,))
+    return s
+
+
+def memory_inputs(row: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], qk: torch.Tensor, *,
+                  heads: int, head_dim: int, q_scale: float = 1.0, k_scale: float = 1.0) -> None:
+    """Queries and keys as a matrix memory's recurrence takes them, in float32: qk[0] = q_scale * rot(q),
+    qk[1] = k_scale * rot(k).  row T [n, at least 2 * heads * head_dim] (may be a band of a wider row)
+    begins with the query heads, then the key heads; rot turns the first 2 * len(inv_freq) elements of
+    every head by position * inv_freq[j], element j paired with j + len(inv_freq) (inv_freq None: nothing
+    turns); qk float32 [2, n, heads * head_dim]."""
+    _need(row.dim() == 2 and row.dtype in _ACT, "row: expected T [n, w]")
+    n, width = row.shape[0], heads * head_dim
+    _band(row, "row", row.dtype, n, row.shape[1])
+    _need(heads > 0 and head_dim > 0 and row.shape[1] >= 2 * width, lambda: f"row: at least {2 * width} columns")
+    _dense(positions, "positions", torch.int32, (n,))
+    if inv_freq is not None:
+        _dense(inv_freq, "inv_freq", torch.float32)
+        _need(inv_freq.dim() == 1 and 0 < 2 * inv_freq.shape[0] <= head_dim,
+              lambda: f"inv_freq: {tuple(inv_freq.shape)} does not fit head_dim {head_dim}")
+    _dense(qk, "qk", torch.float32, (2, n, width))
+    if n:
+        call("memory_inputs", row, positions, inv_freq, qk, heads, head_dim, float(q_scale), float(k_scale))
+
+
+def memory_gates(gates: torch.Tensor, i_bias: Optional[torch.Tensor], f_bias: Optional[torch.Tensor], qk: torch.Tensor,
+                 state: torch.Tensor, carried_offset: int, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
+                 state_slots: torch.Tensor, steps: torch.Tensor, *, heads: int, head_dim: int,
+                 cap: Optional[float] = None, den_eps: float = 1e-6) -> None:
+    """Exponential gates held in range by a running maximum, over each segment's tokens in order.  Per head:
+        i = cap tanh((z_i + i_bias) / cap);  f = logsigmoid(cap tanh((z_f + f_bias) / cap))   (cap None: no cap)
+        m_t = max(f + m_(t-1), i);  a = exp(f + m_(t-1) - m_t);  b = exp(i - m_t)
+        n_t = a n_(t-1) + b k_t;    den = max(|n_t . q_t|, exp(-m_t)) + den_eps
+    gates T [n, 2 * heads] (may be a band): z_i of all heads, then z_f; biases float32 [heads] or None;
+    qk float32 [2, n, heads * head_dim] as `memory_inputs` left it; state float32 [slots, W] holds, from
+    column `carried_offset` of row state_slots[segment], n as [heads, head_dim] and then m as [heads]
+    (zeros for a fresh request); steps float32 [3, n, heads] takes a, b and den.  All float32."""
+    _need(gates.dim() == 2 and gates.dtype in _ACT, "gates: expected T [n, 2 * heads]")
+    n = gates.shape[0]
+    _band(gates, "gates", gates.dtype, n, 2 * heads)
+    _need(0 < head_dim <= 256, "head_dim: from 1 to 256")
+    for t, name in ((i_bias, "i_bias"), (f_bias, "f_bias")):
+        if t is not None:
+            _dense(t, name, torch.float32, (heads,))
+    _dense(qk, "qk", torch.float32, (2, n, heads * head_dim))
+    _dense(state, "state", torch.float32)
+    _need(state.dim() == 2 and 0 <= carried_offset and carried_offset + heads * head_dim + heads <= state.shape[1],
+          "state: a row holds n and m from carried_offset")
+    _segments(seg_q_start, seg_q_len, state_slots)
+    _dense(steps, "steps", torch.float32, (3, n, heads))
+    _need(cap is None or cap > 0, "cap must be positive or None")
+    if n:
+        call("memory_gates", gates, i_bias, f_bias, qk, state, int(carried_offset), seg_q_start, seg_q_len, state_slots,
+             steps, heads, head_dim, cap, float(den_eps))
+
+
+def memory_scan(qk: torch.Tensor, v: torch.Tensor, steps: Optional[torch.Tensor], decays: Optional[torch.Tensor],
+                state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor,
+                y: torch.Tensor, *, heads: int, head_dim: int, value_dim: int) -> None:
+    """The matrix memory's recurrence over each segment's tokens in order, from and into the request's
+    carried state.  Per head:  S = a S + b k v^T;  y = S^T q / den  with (a, b, den) of the token from
+    `steps` (float32 [3, n, heads]) or, with `decays` (float32 [heads]) instead, (decays[h], 1, 1).
+    qk float32 [2, n, heads * head_dim]: queries, then keys; v T [n, heads * value_dim] (may be a band);
+    state float32 [slots, W], whose row state_slots[segment] begins with S as [heads, head_dim, value_dim];
+    y float32 [n, heads * value_dim].  All of the recurrence is float32."""
+    _need((steps is None) != (decays is None), "steps or decays, one of the two")
+    _need(v.dim() == 2 and v.dtype in _ACT, "v: expected T [n, heads * value_dim]")
+    n = v.shape[0]
+    _band(v, "v", v.dtype, n, heads * value_dim)
+    _need(0 < head_dim <= 256 and value_dim > 0, "head_dim: from 1 to 256")
+    _dense(qk, "qk", torch.float32, (2, n, heads * head_dim))
+    if steps is not None:
+        _dense(steps, "steps", torch.float32, (3, n, heads))
+    else:
+        _dense(decays, "decays", torch.float32, (heads,))
+    _dense(state, "state", torch.float32)
+    _need(state.dim() == 2 and state.shape[1] >= heads * head_dim * value_dim, "state: a row holds at least [heads, D, P]")
+    _segments(seg_q_start, seg_q_len, state_slots)
+    _dense(y, "y", torch.float32, (n, heads * value_dim))
+    if n:
+        call("memory_scan", qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads, head_dim, value_dim)
+
+
+def head_norm_gate(y: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], out: torch.Tensor, *, heads: int,
+                   eps: float, activation: str = "sigmoid", scale: float = 1.0) -> None:
+    """out = y / rms_of_its_head(y) * weight * act(gate) * scale: every one of `heads` equal parts of a row
+    of y is divided by sqrt(mean of its squares + eps).  y float32 [n, W]; gate T [n, W] and out T [n, W]
+    may be bands of wider tensors; weight float32 [W] or None; activation "sigmoid" or "silu"."""
+    _need(activation in GATE_KINDS, lambda: f"activation {activation!r}: expected one of {sorted(GATE_KINDS)}")
+    _dense(y, "y", torch.float32)
+    _need(y.dim() == 2 and heads > 0 and y.shape[1] % heads == 0, "y: expected [n, heads * P]")
+    n, w = y.shape
+    _need(gate.dtype in _ACT, "gate: expected T")
+    _band(gate, "gate", gate.dtype, n, w)
+    _band(out, "out", gate.dtype, n, w)
+    if weight is not None:
+        _dense(weight, "weight", torch.float32, (w,))
+    if n:
+        call("head_norm_gate", y, gate, weight, out, heads, float(eps), activation, float(scale))
+
+
+# ---- a mixture of experts ------------------------------------------------------------------------------
+MOE_TILE_ROWS = 16
+MOE_MAX_EXPERTS = 256
+
+
+def moe_max_tiles(assignments: int, experts: int) -> int:
+    """The most tiles of `MOE_TILE_ROWS` rows that `assignments` (token, expert) pairs can fill when the
+    pairs of an expert lie together and every expert's last tile may be partly empty."""
+    return assignments // MOE_TILE_ROWS + experts
+
+
+def moe_plan_size(assignments: int, experts: int) -> int:
+    """int32 elements of the plan `moe_plan` writes: the number of tiles in use, a tile's expert for
+    every tile there is room for, and the rows of every tile."""
+    return 1 + moe_max_tiles(assignments, experts) * (1 + MOE_TILE_ROWS)
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, *, groups: int = 1,
+              keep: int = 1, eps: float = 1e-20) -> None:
+    """Which experts each token uses.  z = x router^T in float32; s = softmax(z) over all experts; the
+    experts form `groups` equal groups of neighbours, a group's score is its largest s, and only experts of
+    the `keep` best groups may be chosen; the `top` = ids.shape[1] allowed experts with the largest s are
+    chosen (of equal scores the lower index first), weights = their s / (sum of the chosen + eps).
+    x T [n, width]; router float32 [experts, width]; ids int32 [n, top]; weights float32 [n, top]."""
+    _dense(x, "x", _ACT)
+    _need(x.dim() == 2, "x: expected [n, width]")
+    n, width = x.shape
+    _dense(router, "router", torch.float32)
+    _need(router.dim() == 2 and router.shape[1] == width and 0 < router.shape[0] <= MOE_MAX_EXPERTS,
+          lambda: f"router: expected [at most {MOE_MAX_EXPERTS} experts, {width}]")
+    experts = router.shape[0]
+    _dense(ids, "ids", torch.int32)
+    _need(ids.dim() == 2 and ids.shape[0] == n, "ids: expected [n, top]")
+    top = ids.shape[1]
+    _dense(weights, "weights", torch.float32, (n, top))
+    _need(groups > 0 and experts % groups == 0 and 0 < keep <= groups, "groups must divide the experts; keep from 1 to groups")
+    _need(0 < top <= keep * (experts // groups), "top: at most the experts of the kept groups")
+    if n:
+        call("moe_route", x, router, ids, weights, int(groups), int(keep), float(eps))
+
+
+def moe_plan(ids: torch.Tensor, plan: torch.Tensor, experts: int) -> None:
+    """Sorts a step's assignments (a = token * top + slot, expert ids.flat[a]) by expert, in tiles of
+    `MOE_TILE_ROWS` rows: plan[0] = tiles in use; plan[1 + t] = expert of tile t; plan[1 + T + 16 t + r] =
+    the assignment in row r of tile t, or -1, with T = moe_max_tiles(ids.numel(), experts).  An expert's
+    assignments lie together in any order.  ids int32 [n, top]; plan int32 [moe_plan_size(...)]."""
+    _dense(ids, "ids", torch.int32)
+    _need(ids.dim() == 2, "ids: expected [n, top]")
+    _need(0 < experts <= MOE_MAX_EXPERTS, f"experts: from 1 to {MOE_MAX_EXPERTS}")
+    _dense(plan, "plan", torch.int32, (moe_plan_size(ids.numel(), experts),))
+    if ids.numel():
+        call("moe_plan", ids, plan, int(experts))
+
+
+def moe_experts_up(x: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, act: torch.Tensor, top: int,
+                   activation: str) -> None:
+    """act[a] = activation(x[a // top] Wg_e^T) * (x[a // top] Wu_e^T) for every assignment a of the plan, e
+    its expert.  x T [n, width]; w T [experts, 2 * ff, width]: an expert's gate rows, then its up rows; act
+    T [n * top, ff]; float32 sums."""
+    _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {sorted(ACTIVATIONS)}")
+    _dense(x, "x", _ACT)
+    _need(x.dim() == 2, "x: expected [n, width]")
+    n, width = x.shape
+    _dense(w, "w", x.dtype)
+    _need(w.dim() == 3 and w.shape[2] == width and w.shape[1] % 2 == 0, "w: expected [experts, 2 * ff, width]")
+    experts, ff = w.shape[0], w.shape[1] // 2
+    _dense(act, "act", x.dtype, (n * top, ff))
+    _dense(plan, "plan", torch.int32, (moe_plan_size(n * top, experts),))
+    if n:
+        call("moe_experts_up", x, w, plan, act, int(top), activation)
+
+
+def moe_experts_down(act: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, weights: torch.Tensor,
+                     out: torch.Tensor) -> None:
+    """out[a % top][a // top] = weights.flat[a] * (act[a] Wd_e^T) for every assignment a of the plan: the
+    experts' weighted results as a stack of `top` float32 partial sums over the tokens.  act T [n * top, ff];
+    w T [experts, width, ff]; weights float32 [n, top]; out float32 [top, n, width]."""
+    _dense(act, "act", _ACT)
+    _need(act.dim() == 2, "act: expected [n * top, ff]")
+    _dense(weights, "weights", torch.float32)
+    _need(weights.dim() == 2 and weights.numel() == act.shape[0], "weights: expected [n, top]")
+    n, top = weights.shape
+    _dense(w, "w", act.dtype)
+    _need(w.dim() == 3 and w.shape[2] == act.shape[1], "w: expected [experts, width, ff]")
+    _dense(out, "out", torch.float32, (top, n, w.shape[1]))
+    _dense(plan, "plan", torch.int32, (moe_plan_size(n * top, w.shape[0]),))
+    if n:
+        call("moe_experts_down", act, w, plan, weights, out)
+
+
 # ---- the framework's own operations that go through the same door as a part's ------------------
 def _register_own() -> None:
     from ctypes import c_float, c_int, c_longlong, c_void_p
@@ -918,10 +1124,10 @@ def _register_own() -> None:
                     p(a), a.stride(0), p(gate), gate.stride(0), p(out), out.stride(0), int(a.dtype == torch.bfloat16),
                     a.shape[0], a.shape[1], per, stream))
     register_op("copy_columns", entry_point="wllm_copy_columns",
-                argtypes=[c_void_p, c_longlong, c_void_p, c_longlong, c_int, c_int, c_int, c_void_p],
-                launch=lambda fn, stream, src, out: fn(
+                argtypes=[c_void_p, c_longlong, c_void_p, c_longlong, c_int, c_int, c_int, c_float, c_void_p],
+                launch=lambda fn, stream, src, out, scale=1.0: fn(
                     p(src), src.stride(0), p(out), out.stride(0), int(src.dtype == torch.bfloat16), src.shape[0],
-                    src.shape[1], stream))
+                    src.shape[1], scale, stream))
 
     def add(fn, stream, x, addend, delta, delta_bias):
         splits, stride = 1, 0
@@ -954,14 +1160,15 @@ def _register_own() -> None:
 
     def band_norm_launch(fn, stream, bands, eps):
         args = []
-        for src, weight, count, out in bands:
-            args += [p(src), src.stride(0), src.shape[1], p(weight), float(count), p(out), out.stride(0), out.shape[1]]
+        for src, weight, count, out, bias in bands:
+            args += [p(src), src.stride(0), src.shape[1], p(weight), float(count), p(out), out.stride(0), out.shape[1],
+                     p(bias)]
         if len(bands) == 1:
-            args += [p(None), 0, 0, p(None), 1.0, p(None), 0, 0]
+            args += [p(None), 0, 0, p(None), 1.0, p(None), 0, 0, p(None)]
         first = bands[0][0]
         return fn(*args, eps, int(first.dtype == torch.bfloat16), first.shape[0], stream)
 
-    one_band = [c_void_p, c_longlong, c_int, c_void_p, c_float, c_void_p, c_longlong, c_int]
+    one_band = [c_void_p, c_longlong, c_int, c_void_p, c_float, c_void_p, c_longlong, c_int, c_void_p]
     register_op("band_norm", entry_point="wllm_band_norm", argtypes=one_band + one_band + [c_float, c_int, c_int, c_void_p],
                 launch=band_norm_launch)
     register_op("gated_lookup", entry_point="wllm_gated_lookup",
@@ -995,6 +1202,55 @@ def _register_own() -> None:
                 launch=lambda fn, stream, y, z, weight, out, groups, eps: fn(
                     p(y), p(z), z.stride(0), p(weight), p(out), int(z.dtype == torch.bfloat16), y.shape[0], y.shape[1],
                     groups, eps, stream))
+
+    bf = lambda t: int(t.dtype == torch.bfloat16)
+    register_op("memory_inputs", entry_point="wllm_memory_inputs",
+                argtypes=[c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
+                          c_float, c_void_p],
+                launch=lambda fn, stream, row, positions, inv_freq, qk, heads, head_dim, q_scale, k_scale: fn(
+                    p(row), row.stride(0), p(positions), p(inv_freq), p(qk), bf(row), row.shape[0], heads, head_dim,
+                    2 * inv_freq.shape[0] if inv_freq is not None else 0, q_scale, k_scale, stream))
+    register_op("memory_gates", entry_point="wllm_memory_gates",
+                argtypes=[c_void_p, c_longlong, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_longlong,
+                          c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, gates, i_bias, f_bias, qk, state, carried_offset, seg_q_start, seg_q_len,
+                state_slots, steps, heads, head_dim, cap, den_eps: fn(
+                    p(gates), gates.stride(0), p(i_bias), p(f_bias), float(cap) if cap else 0.0, den_eps, p(qk), p(state),
+                    state.stride(0), carried_offset, p(seg_q_start), p(seg_q_len), p(state_slots), p(steps), bf(gates),
+                    gates.shape[0], seg_q_start.shape[0], heads, head_dim, stream))
+    register_op("memory_scan", entry_point="wllm_memory_scan",
+                argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p,
+                          c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads,
+                head_dim, value_dim: fn(
+                    p(qk), p(v), v.stride(0), p(steps), p(decays), p(state), state.stride(0), p(seg_q_start), p(seg_q_len),
+                    p(state_slots), p(y), bf(v), v.shape[0], seg_q_start.shape[0], heads, head_dim, value_dim, stream))
+    register_op("head_norm_gate", entry_point="wllm_head_norm_gate",
+                argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int,
+                          c_float, c_float, c_void_p],
+                launch=lambda fn, stream, y, gate, weight, out, heads, eps, activation, scale: fn(
+                    p(y), p(gate), gate.stride(0), p(weight), p(out), out.stride(0), bf(gate), GATE_KINDS[activation],
+                    y.shape[0], heads, y.shape[1] // heads, eps, scale, stream))
+    register_op("moe_route", entry_point="wllm_moe_route",
+                argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                          c_void_p],
+                launch=lambda fn, stream, x, router, ids, weights, groups, keep, eps: fn(
+                    p(x), p(router), p(ids), p(weights), bf(x), x.shape[0], x.shape[1], router.shape[0], ids.shape[1], groups,
+                    keep, eps, stream))
+    register_op("moe_plan", entry_point="wllm_moe_plan", argtypes=[c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, ids, plan, experts: fn(
+                    p(ids), p(plan), ids.numel(), experts, moe_max_tiles(ids.numel(), experts), stream))
+    register_op("moe_experts_up", entry_point="wllm_moe_up",
+                argtypes=[c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, x, w, plan, act, top, activation: fn(
+                    p(x), p(w), p(plan), moe_max_tiles(act.shape[0], w.shape[0]), p(act), bf(x), ACTIVATIONS[activation],
+                    x.shape[1], act.shape[1], top, stream))
+    register_op("moe_experts_down", entry_point="wllm_moe_down",
+                argtypes=[c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                          c_void_p],
+                launch=lambda fn, stream, act, w, plan, weights, out: fn(
+                    p(act), p(w), p(plan), moe_max_tiles(act.shape[0], w.shape[0]), p(weights), p(out), bf(act),
+                    weights.shape[0], act.shape[1], w.shape[1], weights.shape[1], stream))
 
 
 _register_own()

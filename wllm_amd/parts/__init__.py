@@ -1,5 +1,5 @@
-from wllm_amd.parts import (attention, blocks, feed_forward, latent_attention, norms, positions,  # noqa: F401
-                            state_space)                                                     # (register the kinds)
+from wllm_amd.parts import (attention, blocks, feed_forward, latent_attention, matrix_memory,  # noqa: F401
+                            mixture_of_experts, norms, positions, side_by_side, state_space)  # (register the kinds)
 from wllm_amd.parts.model import (CausalLM, build_model, load_model, resolve_dtype, write_random_model_folder,
                                    write_random_model_from_config_json)
 from wllm_amd.parts.registry import (

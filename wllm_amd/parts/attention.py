@@ -46,7 +46,8 @@ class PagedAttention:
             raise ValueError(f"window must be positive or None, got {spec.window}")
         plain = not (spec.softcap or spec.qk_norm_eps is not None or spec.values_are_keys or spec.gate_weight
                      or spec.position.pairing == "interleaved" or spec.value_dim not in (None, spec.head_dim)
-                     or spec.chunk or spec.q_norm_weight or spec.k_norm_weight or not spec.owns_cache)
+                     or spec.chunk or spec.q_norm_weight or spec.k_norm_weight or not spec.owns_cache
+                     or spec.sink is not None or spec.output_scale != 1.0)
         if spec.chunk is not None and (spec.chunk <= 0 or spec.window is not None):
             raise ValueError(f"chunk must be positive and excludes a window, got chunk {spec.chunk}, window {spec.window}")
         if (spec.q_norm_weight or spec.k_norm_weight) and spec.band_norm_eps is None:
@@ -55,6 +56,8 @@ class PagedAttention:
                                     or spec.qk_norm_eps is not None or spec.position.kind != "none"):
             raise ValueError("a layer without a cache of its own has no key or value projection, and its queries "
                              "are neither rotated nor normed head by head")
+        if spec.bias_before_norm and not (spec.q_norm_weight and (spec.k_norm_weight or not spec.owns_cache)):
+            raise ValueError("bias_before_norm: the query and key projections have norms over the whole projection")
         if spec.gate_per_head and not spec.gate_weight:
             raise ValueError("gate_per_head without a gate")
         if (plain and spec.head_dim % ops.HEAD_DIM_STEP) or not 0 < spec.head_dim <= ops.MAX_HEAD_DIM:
@@ -84,6 +87,8 @@ class PagedAttention:
         if not 0 < self.dim <= ops.MAX_HEAD_DIM:
             raise ValueError(f"value_dim {self.vdim}: the attention kernels take heads up to {ops.MAX_HEAD_DIM}")
         self.w_q_norm = self.w_k_norm = None
+        self.b_q = self.b_k = None          # biases that are added in front of the norm over a whole projection
+        self.sinks = None
 
     @property
     def qkv_width(self) -> int:
@@ -122,7 +127,7 @@ class PagedAttention:
             out[s.q_norm_weight] = ExpectedTensor((q,), role="vector", init="norm")
         if s.k_norm_weight and s.owns_cache:
             out[s.k_norm_weight] = ExpectedTensor((kv,), role="vector", init="norm")
-        for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, kv), (s.o_bias, s.hidden_size)):
+        for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, s.num_kv_heads * self.vdim), (s.o_bias, s.hidden_size)):
             if name is not None:
                 out[name] = ExpectedTensor((width,), role="vector")
         if hasattr(self.position, "expected_tensors"):      # a position encoding with tensors of its own
@@ -164,15 +169,25 @@ class PagedAttention:
             self.b_o = fetch.to_device(fetch.vector(s.o_bias))
         if s.q_bias is not None or s.k_bias is not None or s.v_bias is not None:
             q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
-            if self.vdim != s.head_dim or not s.owns_cache:
-                raise NotImplementedError("biases of the projections beside value heads of another size")
-            biases = [(s.q_bias, q), (s.k_bias, kv)] + ([] if s.values_are_keys else [(s.v_bias, kv)])
+            if not s.owns_cache:
+                raise NotImplementedError("biases of the projections of a layer without keys of its own")
+            biases = [(s.q_bias, q, s.head_dim), (s.k_bias, kv, s.head_dim)]
+            biases += [] if s.values_are_keys else [(s.v_bias, s.num_kv_heads * self.vdim, self.vdim)]
             # (the gate's projection, behind the heads in the row, has none: the bias is shorter than the row)
-            found = [fetch.vector(name) if name is not None else None for name, _ in biases]
+            found = [fetch.vector(name) if name is not None else None for name, _, _ in biases]
             where = next(v.device for v in found if v is not None)      # a fetcher may make its tensors on the device
-            parts = [heads_padded(v if v is not None else torch.zeros(width, device=where), 0)
-                     for v, (_, width) in zip(found, biases)]
-            self.b_qkv = fetch.to_device(torch.cat(parts))
+            parts = [heads_padded(v if v is not None else torch.zeros(width, device=where), 0, size)
+                     for v, (_, width, size) in zip(found, biases)]
+            if s.bias_before_norm:
+                # the norm kernel adds the queries' and keys' biases as it reads; what is left for the
+                # kernel behind it is the values' bias
+                self.b_q = fetch.to_device(parts[0]) if s.q_bias is not None else None
+                self.b_k = fetch.to_device(parts[1]) if s.k_bias is not None else None
+                parts[0], parts[1] = torch.zeros_like(parts[0]), torch.zeros_like(parts[1])
+            if not s.bias_before_norm or (len(parts) > 2 and s.v_bias is not None):
+                self.b_qkv = fetch.to_device(torch.cat(parts))
+        if s.sink is not None:
+            self.sinks = torch.full((s.num_heads,), float(s.sink), dtype=torch.float32, device=fetch.device)
         if hasattr(self.position, "load"):
             self.position.load(fetch)
         self.position.prepare(fetch.device)
@@ -237,10 +252,10 @@ class PagedAttention:
             q_width, kv_width = s.num_heads * self.dim, s.num_kv_heads * self.dim
             bands = []
             if self.w_q_norm is not None:
-                bands.append((qkv[:, :q_width], self.w_q_norm, s.num_heads * s.head_dim, qkv[:, :q_width]))
+                bands.append((qkv[:, :q_width], self.w_q_norm, s.num_heads * s.head_dim, qkv[:, :q_width], self.b_q))
             if self.w_k_norm is not None:
                 bands.append((qkv[:, q_width:q_width + kv_width], self.w_k_norm, s.num_kv_heads * s.head_dim,
-                              qkv[:, q_width:q_width + kv_width]))
+                              qkv[:, q_width:q_width + kv_width], self.b_k))
             if bands:
                 ops.band_norm(bands, s.band_norm_eps)
             if s.owns_cache:
@@ -287,15 +302,18 @@ class PagedAttention:
             page_size=pages.page_size, scale=s.scale, window=s.window or 0,
             max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len,
             plan=self._work_items(ctx, pages.page_size), softcap=s.softcap or 0.0, exact_weights=s.weights_in_float32,
-            chunk=s.chunk or 0)
+            chunk=s.chunk or 0, sinks=self.sinks)
         if s.gate_weight:
             # the gate's columns lie behind the heads in the projected row
             gate = qkv[:, self.gate_offset:self.gate_offset + self.gate_width]
             target = product_input if product_input is not None else attn
             ops.sigmoid_gate(attn, gate, target, per=self.dim if s.gate_per_head else 1)
             attn = target
-        elif product_input is not None:
-            ops.copy_columns(attn, product_input)
-            attn = product_input
+            if s.output_scale != 1.0:
+                ops.copy_columns(attn, attn, s.output_scale)
+        elif product_input is not None or s.output_scale != 1.0:
+            target = product_input if product_input is not None else attn
+            ops.copy_columns(attn, target, s.output_scale)
+            attn = target
         # the stream adds the output projection: at once, or through the next norm, partial sums and all
         return Product("mixer_out", attn, self.w_o, self.t_o, bias=self.b_o)

@@ -136,16 +136,24 @@ class PreNormBlock:
     def __init__(self, spec: BlockSpec):
         self.spec = spec
         self.mixer = build_mixer(spec.mixer)
-        self.feed_forward = build_feed_forward(spec.feed_forward)
         self.mixer_norm = build_norm(spec.mixer_norm)
-        self.feed_forward_norm = build_norm(spec.feed_forward_norm)
+        # a layer may be its mixer alone
+        self.feed_forward = self.feed_forward_norm = None
+        if spec.feed_forward is not None:
+            if spec.feed_forward_norm is None:
+                raise ValueError("a pre-norm block's feed-forward has a norm before it")
+            self.feed_forward = build_feed_forward(spec.feed_forward)
+            self.feed_forward_norm = build_norm(spec.feed_forward_norm)
 
     def parts(self) -> list:
-        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+        own = [self.mixer_norm, self.mixer]
+        return own + ([self.feed_forward_norm, self.feed_forward] if self.feed_forward is not None else [])
 
     def forward(self, ctx, entry: int, stream: ResidualStream) -> None:
         h = stream.input_for(ctx, self.mixer_norm, self.mixer)
         stream.add(ctx, self.mixer.forward(ctx, entry, h))
+        if self.feed_forward is None:
+            return
         h = stream.input_for(ctx, self.feed_forward_norm, self.feed_forward)
         stream.add(ctx, self.feed_forward.forward(ctx, h))
 

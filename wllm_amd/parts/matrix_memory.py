@@ -1,0 +1,141 @@
+"""A recurrent mixer whose state is a matrix a head: linear attention in its recurrent form.
+
+    [q | k | v | g | (z_i | z_f)] = W h                one stacked product
+    q = q_scale * rot(q),  k = k_scale * rot(k)        float32 from here on (rot: the spec's position, or none)
+    S_t = a_t S_(t-1) + b_t k_t v_t^T                  per head, S [head_dim, value_dim], float32
+    o_t = S_t^T q_t / den_t
+    out = W_o (o / rms_per_head(o) * w * act(g) * output_scale)
+
+With `gating` "decay", a_t is the head's fixed decay and b_t = den_t = 1 (retention).  With "exponential",
+the two gate projections give a log input gate and a log forget gate (both bent under a cap), a running
+maximum m holds the exponentials in range, a normaliser n_t = a_t n_(t-1) + b_t k_t is carried beside S and
+den_t = max(|n_t . q_t|, exp(-m_t)) + den_eps (the matrix memory of an mLSTM).
+
+A request carries S (and n, m) from step to step in one float32 state row of the cache manager
+([heads * head_dim * value_dim], then [heads * head_dim], then [heads]; zeroed at admission: all three
+start at zero).  The kernels walk every segment's tokens in order from that row and leave it for the
+next step, so a prompt may be cut anywhere, and a decoded token is a segment of one.  Everything the
+kernels read of the step lies in device arrays, so a decode step can be captured in a graph.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from wllm_amd.kernels import ops
+from wllm_amd.parts.common import Product, load_matrix
+from wllm_amd.parts.registry import build_position, register_mixer
+from wllm_amd.parts.specs import MatrixMemorySpec
+from wllm_amd.weights.checkpoint import ExpectedTensor
+
+
+@register_mixer("matrix_memory")
+class MatrixMemoryMixer:
+    graph_capturable = True
+
+    def __init__(self, spec: MatrixMemorySpec):
+        for name in ("hidden_size", "num_heads", "head_dim", "value_dim"):
+            if getattr(spec, name) <= 0:
+                raise ValueError(f"{name} must be positive, got {getattr(spec, name)}")
+        if spec.head_dim > 256:
+            raise ValueError(f"head_dim {spec.head_dim}: the recurrence's kernel keeps at most 256 rows a head")
+        if spec.gating not in ("decay", "exponential"):
+            raise ValueError(f"gating {spec.gating!r}: 'decay' or 'exponential'")
+        if spec.gating == "decay" and len(spec.decays) != spec.num_heads:
+            raise ValueError(f"decays: one a head ({spec.num_heads}), got {len(spec.decays)}")
+        if spec.gating == "exponential" and not (spec.i_weight and spec.f_weight):
+            raise ValueError("exponential gating needs the two gate projections")
+        if spec.gate_cap is not None and not spec.gate_cap > 0:
+            raise ValueError(f"gate_cap must be positive or None, got {spec.gate_cap}")
+        if spec.gate_activation not in ops.GATE_KINDS:
+            raise ValueError(f"gate_activation {spec.gate_activation!r}: one of {sorted(ops.GATE_KINDS)}")
+        if spec.position.kind == "rope" and (spec.position.pairing != "half" or spec.position.rotary_dim > spec.head_dim):
+            raise ValueError("the rotation pairs element j with j + rotary_dim / 2, within the head")
+        self.spec = spec
+        self.position = build_position(spec.position)
+        self.exponential = spec.gating == "exponential"
+        self.qk_width = spec.num_heads * spec.head_dim
+        self.v_width = spec.num_heads * spec.value_dim
+        self.v_offset = 2 * self.qk_width
+        self.g_offset = self.v_offset + self.v_width
+        self.gates_offset = self.g_offset + self.v_width
+        width = self.gates_offset + (2 * spec.num_heads if self.exponential else 0)
+        self.in_width = -(-width // 8) * 8             # rows of the stacked weight, padded with zero rows
+        self.memory_size = spec.num_heads * spec.head_dim * spec.value_dim
+        self.w_in = self.t_in = self.w_o = self.t_o = None
+        self.norm_w = self.i_bias = self.f_bias = self.decays = None
+
+    def expected_tensors(self) -> dict:
+        s = self.spec
+        out = {
+            s.q_weight: ExpectedTensor((self.qk_width, s.hidden_size)),
+            s.k_weight: ExpectedTensor((self.qk_width, s.hidden_size)),
+            s.v_weight: ExpectedTensor((self.v_width, s.hidden_size)),
+            s.gate_weight: ExpectedTensor((self.v_width, s.hidden_size)),
+            s.o_weight: ExpectedTensor((s.hidden_size, self.v_width)),
+        }
+        if s.norm_weight:
+            out[s.norm_weight] = ExpectedTensor((self.v_width,), role="vector", init="norm")
+        if self.exponential:
+            out[s.i_weight] = ExpectedTensor((s.num_heads, s.hidden_size))
+            out[s.f_weight] = ExpectedTensor((s.num_heads, s.hidden_size))
+            for name in (s.i_bias, s.f_bias):
+                if name:
+                    out[name] = ExpectedTensor((s.num_heads,), role="vector")
+        return out
+
+    def load(self, fetch) -> None:
+        s = self.spec
+        stacked = [fetch.matrix(name) for name in (s.q_weight, s.k_weight, s.v_weight, s.gate_weight)]
+        if self.exponential:
+            stacked += [fetch.matrix(s.i_weight), fetch.matrix(s.f_weight)]
+        w = torch.cat(stacked, dim=0)
+        if w.shape[0] < self.in_width:
+            w = torch.cat([w, torch.zeros(self.in_width - w.shape[0], w.shape[1], dtype=w.dtype, device=w.device)], dim=0)
+        self.w_in, self.t_in = load_matrix(fetch, w)
+        self.w_o, self.t_o = load_matrix(fetch, fetch.matrix(s.o_weight))
+        # everything that enters the recurrence is kept in float32
+        if s.norm_weight:
+            self.norm_w = fetch.to_device(fetch.vector(s.norm_weight))
+        if self.exponential:
+            self.i_bias = fetch.to_device(fetch.vector(s.i_bias)) if s.i_bias else None
+            self.f_bias = fetch.to_device(fetch.vector(s.f_bias)) if s.f_bias else None
+        else:
+            self.decays = torch.tensor([float(d) for d in s.decays], dtype=torch.float32, device=fetch.device)
+        self.position.prepare(fetch.device)
+
+    def cache_need(self):
+        return None
+
+    def state_shape(self):
+        s = self.spec
+        return (self.memory_size + ((s.num_heads * s.head_dim + s.num_heads) if self.exponential else 0),)
+
+    def flops(self, tokens: int, keys: float = 0.0) -> float:
+        s = self.spec
+        return 2.0 * tokens * (s.hidden_size * (self.in_width + self.v_width) + 2 * self.memory_size)
+
+    def forward(self, ctx, entry: int, h: torch.Tensor, product_input: Optional[torch.Tensor] = None):
+        s = self.spec
+        n = h.shape[0]
+        row = ctx.buffer("memory_in", (n, self.in_width), h.dtype)
+        ops.linear(h, self.w_in, row, self.t_in)
+        state = ctx.state(entry)
+        qk = ctx.buffer("memory_qk", (2, n, self.qk_width), torch.float32)
+        ops.memory_inputs(row, ctx.positions, self.position.inv_freq, qk, heads=s.num_heads, head_dim=s.head_dim,
+                          q_scale=s.q_scale, k_scale=s.k_scale)
+        steps = None
+        if self.exponential:
+            steps = ctx.buffer("memory_steps", (3, n, s.num_heads), torch.float32)
+            ops.memory_gates(row[:, self.gates_offset:self.gates_offset + 2 * s.num_heads], self.i_bias, self.f_bias, qk,
+                             state, self.memory_size, ctx.seg_q_start, ctx.seg_q_len, ctx.state_slots, steps,
+                             heads=s.num_heads, head_dim=s.head_dim, cap=s.gate_cap, den_eps=s.den_eps)
+        y = ctx.buffer("memory_y", (n, self.v_width), torch.float32)
+        ops.memory_scan(qk, row[:, self.v_offset:self.v_offset + self.v_width], steps, self.decays, state,
+                        ctx.seg_q_start, ctx.seg_q_len, ctx.state_slots, y, heads=s.num_heads, head_dim=s.head_dim,
+                        value_dim=s.value_dim)
+        out = product_input if product_input is not None else ctx.buffer("memory_out", (n, self.v_width), h.dtype)
+        ops.head_norm_gate(y, row[:, self.g_offset:self.g_offset + self.v_width], self.norm_w, out, heads=s.num_heads,
+                           eps=s.norm_eps, activation=s.gate_activation, scale=s.output_scale)
+        return Product("mixer_out", out, self.w_o, self.t_o)

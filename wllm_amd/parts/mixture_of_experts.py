@@ -1,0 +1,92 @@
+"""A mixture of gated feed-forward experts of which every token uses a few.
+
+    z = W_router x (float32);  s = softmax(z) over all experts
+    only experts of the `keep_groups` best of `num_groups` groups of neighbours may be chosen
+    the `top` allowed experts with the largest s; weights s / (sum of the chosen + weight_eps)
+    y = sum over the chosen e of weight_e * down_e(act(gate_e(x)) * up_e(x))
+
+The experts' matrices are stacked at load ([experts, 2 * ff, width]: an expert's gate rows, then its up
+rows; [experts, width, ff]).  A step routes its tokens, sorts the (token, expert) pairs by expert on the
+device (`ops.moe_plan`: tiles of 16 rows of one expert) and runs the two products expert by expert on
+the matrix cores, each tile with its expert's weights.  The second product weighs a pair's result and
+leaves it in the slice of its slot of a float32 stack [top, tokens, width], which whoever adds the
+feed-forward to the stream (the next norm kernel) adds in order: the weighted sum is formed in float32
+and takes no pass of its own.  Nothing of the routing is read on the host.
+"""
+from __future__ import annotations
+
+import torch
+
+from wllm_amd.kernels import ops
+from wllm_amd.parts.registry import register_feed_forward
+from wllm_amd.parts.specs import MixtureOfExpertsSpec
+from wllm_amd.weights.checkpoint import ExpectedTensor
+
+
+@register_feed_forward("mixture_of_experts")
+class MixtureOfExperts:
+    def __init__(self, spec: MixtureOfExpertsSpec):
+        if spec.activation not in ops.ACTIVATIONS:
+            raise ValueError(f"activation {spec.activation!r} is not implemented; known: {ops.ACTIVATIONS}")
+        if not 0 < spec.num_experts <= ops.MOE_MAX_EXPERTS:
+            raise ValueError(f"num_experts {spec.num_experts}: from 1 to {ops.MOE_MAX_EXPERTS}")
+        if spec.num_groups <= 0 or spec.num_experts % spec.num_groups or not 0 < spec.keep_groups <= spec.num_groups:
+            raise ValueError(f"num_groups ({spec.num_groups}) must divide num_experts ({spec.num_experts}), and "
+                             f"keep_groups ({spec.keep_groups}) lie between 1 and num_groups")
+        if not 0 < spec.top <= spec.keep_groups * (spec.num_experts // spec.num_groups):
+            raise ValueError(f"top ({spec.top}): at most the experts of the kept groups")
+        self.spec = spec
+        self.w_router = self.w_up = self.w_down = None
+
+    def _names(self, e: int) -> tuple:
+        s = self.spec
+        p = f"{s.expert_prefix}{e}."
+        return p + s.gate_name, p + s.up_name, p + s.down_name
+
+    def expected_tensors(self) -> dict:
+        s = self.spec
+        # the router works in float32: its weight is kept so (exact from a bfloat16 file)
+        out = {s.router_weight: ExpectedTensor((s.num_experts, s.hidden_size), role="vector")}
+        for e in range(s.num_experts):
+            gate, up, down = self._names(e)
+            out[gate] = ExpectedTensor((s.intermediate_size, s.hidden_size))
+            out[up] = ExpectedTensor((s.intermediate_size, s.hidden_size))
+            out[down] = ExpectedTensor((s.hidden_size, s.intermediate_size))
+        return out
+
+    def load(self, fetch) -> None:
+        s = self.spec
+        ups, downs = [], []
+        for e in range(s.num_experts):
+            gate, up, down = self._names(e)
+            ups.append(torch.cat([fetch.matrix(gate), fetch.matrix(up)], dim=0))
+            downs.append(fetch.matrix(down))
+        self.w_up = fetch.to_device(torch.stack(ups).contiguous())
+        self.w_down = fetch.to_device(torch.stack(downs).contiguous())
+        self.w_router = fetch.to_device(fetch.vector(s.router_weight))
+
+    def flops(self, tokens: int) -> float:
+        s = self.spec
+        return 2.0 * tokens * s.hidden_size * (3 * s.top * s.intermediate_size + s.num_experts)
+
+    def bytes_read(self, tokens: int) -> float:
+        """Bytes of expert weights a step of `tokens` tokens reads at most (every chosen expert once)."""
+        s = self.spec
+        used = min(s.num_experts, tokens * s.top)
+        return 3.0 * used * s.intermediate_size * s.hidden_size * self.w_up.element_size()
+
+    def forward(self, ctx, h, product_input=None):
+        if product_input is not None:
+            raise NotImplementedError("a mixture of experts ends in a product a token and expert, not in one product")
+        s = self.spec
+        n = h.shape[0]
+        ids = ctx.buffer("moe_ids", (n, s.top), torch.int32)
+        weights = ctx.buffer("moe_weights", (n, s.top), torch.float32)
+        ops.moe_route(h, self.w_router, ids, weights, groups=s.num_groups, keep=s.keep_groups, eps=s.weight_eps)
+        plan = ctx.buffer("moe_plan", (ops.moe_plan_size(n * s.top, s.num_experts),), torch.int32)
+        ops.moe_plan(ids, plan, s.num_experts)
+        act = ctx.buffer("moe_act", (n * s.top, s.intermediate_size), h.dtype)
+        ops.moe_experts_up(h, self.w_up, plan, act, s.top, s.activation)
+        out = ctx.buffer("moe_out", (s.top, n, s.hidden_size), torch.float32)
+        ops.moe_experts_down(act, self.w_down, plan, weights, out)
+        return out

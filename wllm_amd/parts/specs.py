@@ -66,7 +66,11 @@ class AttentionSpec(MixerSpec):
     (all heads at once) and over the whole key projection, before the heads are split.
     `gate_per_head`: the gate's projection has one row a head, and its sigmoid multiplies the whole head.
     `owns_cache` False: the layer has no key and value projections (nor their norms); it reads the cache
-    of the schedule entry its run names."""
+    of the schedule entry its run names.  `sink`: the softmax's denominator holds exp(sink) once more for
+    every head, a term with no key and no value (0.0: one is added to the sum of exponentials).
+    `bias_before_norm`: the biases of the query and key projections are added before the norm over the
+    whole projection, not behind it.  `output_scale`: the concatenated heads are multiplied by it before
+    the output projection (a mixer whose result enters a weighted sum with another's)."""
     kind: str = "attention"
     hidden_size: int = 0
     num_heads: int = 0
@@ -96,6 +100,9 @@ class AttentionSpec(MixerSpec):
     band_norm_eps: Optional[float] = None
     gate_per_head: bool = False
     owns_cache: bool = True
+    sink: Optional[float] = None
+    bias_before_norm: bool = False
+    output_scale: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -153,6 +160,56 @@ class StateSpaceSpec(MixerSpec):
 
 
 @dataclass(frozen=True)
+class MatrixMemorySpec(MixerSpec):
+    """A recurrent mixer whose state is a matrix a head, S [head_dim, value_dim] in float32, written by outer
+    products of keys and values and read by queries (linear attention in its recurrent form):
+        q = q_scale * rot(W_q h),  k = k_scale * rot(W_k h),  v = W_v h            (rot: `position`, or none)
+        S_t = a_t S_(t-1) + b_t k_t v_t^T,        o_t = S_t^T q_t / den_t
+    `gating` "decay": a_t is the head's fixed number of `decays`, b_t = den_t = 1 (retention).
+    `gating` "exponential": per head a log input gate i = cap tanh((W_i h + b_i) / cap) and a log forget gate
+    f = logsigmoid(cap tanh((W_f h + b_f) / cap)) (`gate_cap` None: no cap), held in range by a running maximum
+    m_t = max(f + m_(t-1), i) that starts at 0: a_t = exp(f + m_(t-1) - m_t), b_t = exp(i - m_t); a normaliser
+    n_t = a_t n_(t-1) + b_t k_t; den_t = max(|n_t . q_t|, exp(-m_t)) + `den_eps` (the matrix memory of an mLSTM).
+    Then every head's o is divided by its root mean square (`norm_eps` inside the root), the heads are
+    concatenated, multiplied by `norm_weight` (if named), by act(W_g h) with `gate_activation` "sigmoid" or
+    "silu", by `output_scale`, and projected by W_o.  A request carries S (and n, m) from token to token."""
+    kind: str = "matrix_memory"
+    hidden_size: int = 0
+    num_heads: int = 0
+    head_dim: int = 0
+    value_dim: int = 0
+    gating: str = "decay"
+    decays: tuple = ()
+    gate_cap: Optional[float] = None
+    den_eps: float = 1e-6
+    q_scale: float = 1.0
+    k_scale: float = 1.0
+    position: PositionSpec = field(default_factory=lambda: PositionSpec(kind="none"))
+    norm_eps: float = 1e-6
+    norm_weight: Optional[str] = None
+    gate_activation: str = "sigmoid"
+    output_scale: float = 1.0
+    q_weight: str = ""
+    k_weight: str = ""
+    v_weight: str = ""
+    gate_weight: str = ""
+    o_weight: str = ""
+    i_weight: Optional[str] = None
+    i_bias: Optional[str] = None
+    f_weight: Optional[str] = None
+    f_bias: Optional[str] = None
+
+
+@dataclass(frozen=True)
+class SideBySideSpec(MixerSpec):
+    """Two mixers that read the same input; the result is the sum of theirs (each weighs its own with its
+    `output_scale`).  At most one of the two pages a cache and at most one carries a state."""
+    kind: str = "side_by_side"
+    left: MixerSpec = field(default_factory=MixerSpec)
+    right: MixerSpec = field(default_factory=MixerSpec)
+
+
+@dataclass(frozen=True)
 class TokenSideSpec:
     """A per-layer token input behind the feed-forward: e = table[token][offset : offset + dim];
     g = act(W_gate x) * e; y = W_proj g; x += rms(y) * w_norm.  The table [vocab, D] is shared by
@@ -188,10 +245,35 @@ class GatedMLPSpec(FeedForwardSpec):
 
 
 @dataclass(frozen=True)
+class MixtureOfExpertsSpec(FeedForwardSpec):
+    """`num_experts` gated feed-forwards without biases, down_e(act(gate_e(x)) * up_e(x)), of which a token
+    uses `top`.  Router: z = W_router x in float32, s = softmax(z) over all experts.  The experts form
+    `num_groups` equal groups of neighbours; a group's score is its largest s, and only experts of the
+    `keep_groups` best groups can be chosen (one group, one kept: no limit).  The `top` allowed experts with
+    the largest s are chosen, their weights are their s divided by the sum of the chosen (+ `weight_eps`),
+    and the result is the weighted sum of their outputs.  `expert_prefix` + "<e>." + `gate_name` ... name an
+    expert's tensors."""
+    kind: str = "mixture_of_experts"
+    hidden_size: int = 0
+    intermediate_size: int = 0
+    num_experts: int = 0
+    top: int = 1
+    num_groups: int = 1
+    keep_groups: int = 1
+    weight_eps: float = 1e-20
+    activation: str = "silu"
+    router_weight: str = ""
+    expert_prefix: str = ""
+    gate_name: str = "gate"
+    up_name: str = "up"
+    down_name: str = "down"
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One layer: a mixer and a feed-forward with their norms, and how they are
     arranged around the residual stream.  "pre_norm": x += mixer(norm(x));
-    x += ffn(norm(x)).  "parallel": h = mixer_norm(x); x += mixer(h) + ffn(h): one norm, both
+    x += ffn(norm(x)) (`feed_forward` and its norm may be None: then the layer is its mixer alone).  "parallel": h = mixer_norm(x); x += mixer(h) + ffn(h): one norm, both
     sublayers read it (`feed_forward_norm` is None, and `feed_forward` may be None: then the
     layer is its mixer alone).  "sandwich": x += post(mixer(pre(x))); x += post(ffn(pre(x))) with the
     two norms behind the sublayers in `mixer_post_norm` and `feed_forward_post_norm` (a layer without a
