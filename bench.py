@@ -234,7 +234,7 @@ def run_compare(args) -> dict:
                 k = max(8, args.steps // 2)
                 d, ctx_len = measure_decode(model, batch, args.context, k, 4, args.block_size, graphs)
                 state = 2 * model.state_bytes() if hasattr(model, "state_bytes") else 0     # read and written a step
-                gbs = (model.weight_bytes() + batch * (ctx_len * kv_bytes_per_token(model) + state)) / (d / k) / 1e9
+                gbs = (model.weight_bytes(batch) + batch * (ctx_len * kv_bytes_per_token(model) + state)) / (d / k) / 1e9
                 points[f"{key}_decode_b{batch}"] = round(k * batch / d, 1)
                 points[f"{key}_decode_b{batch}_ms"] = round(1000.0 * d / k, 4)
                 points[f"{key}_decode_b{batch}_frac"] = round(gbs / PEAK_HBM_GBS, 4)

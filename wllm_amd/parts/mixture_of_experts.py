@@ -25,6 +25,8 @@ from wllm_amd.weights.checkpoint import ExpectedTensor
 
 @register_feed_forward("mixture_of_experts")
 class MixtureOfExperts:
+    routed_tensors = ("w_up", "w_down")      # a step reads the chosen experts' share of these: `bytes_read`
+
     def __init__(self, spec: MixtureOfExpertsSpec):
         if spec.activation not in ops.ACTIVATIONS:
             raise ValueError(f"activation {spec.activation!r} is not implemented; known: {ops.ACTIVATIONS}")

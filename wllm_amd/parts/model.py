@@ -136,17 +136,30 @@ class CausalLM:
             total += math.prod(dims) * size
         return total
 
-    def weight_bytes(self) -> int:
-        """Bytes of every weight a step reads once (the tied table counts once)."""
+    def weight_bytes(self, tokens: int = None) -> int:
+        """Bytes of every weight a step reads once (the tied table counts once).  A part whose step reads only
+        some of its weights (experts of which a token uses a few) names those in `routed_tensors` and says in
+        `bytes_read(tokens)` how much of them a step of `tokens` tokens reads at most; without `tokens` they
+        count whole."""
         seen, total = set(), 0
         tensors = [self.embed_table if self.head_weight is not self.embed_table else None, self.head_weight,
                    self.final_norm.weight]
+
+        def collect(part):
+            nonlocal total
+            routed = getattr(part, "routed_tensors", ()) if tokens is not None else ()
+            if routed:
+                total += int(part.bytes_read(tokens))
+            # a tile-major copy (t_*) holds the same numbers as its matrix; a step reads one of the two
+            # (nor a table of which a step reads one row a token: the part names it in `lookup_tables`)
+            tensors.extend(v for k, v in vars(part).items() if isinstance(v, torch.Tensor) and not k.startswith("t_")
+                           and k not in getattr(part, "lookup_tables", ()) and k not in routed)
+            for inner in getattr(part, "sub_parts", lambda: ())():
+                collect(inner)
+
         for block in self.blocks:
             for part in block.parts():
-                # a tile-major copy (t_*) holds the same numbers as its matrix; a step reads one of the two
-                # (nor a table of which a step reads one row a token: the part names it in `lookup_tables`)
-                tensors.extend(v for k, v in vars(part).items() if isinstance(v, torch.Tensor) and not k.startswith("t_")
-                               and k not in getattr(part, "lookup_tables", ()))
+                collect(part)
         for t in tensors:
             if t is not None and t.data_ptr() not in seen:
                 seen.add(t.data_ptr())

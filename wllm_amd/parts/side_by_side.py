@@ -36,6 +36,9 @@ class SideBySideMixer:
     def graph_capturable(self) -> bool:
         return getattr(self.left, "graph_capturable", False) and getattr(self.right, "graph_capturable", False)
 
+    def sub_parts(self) -> tuple:
+        return (self.left, self.right)
+
     def expected_tensors(self) -> dict:
         return {**self.left.expected_tensors(), **self.right.expected_tensors()}
 
