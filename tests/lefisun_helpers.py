@@ -214,3 +214,39 @@ def requests_for(name, lengths) -> dict:
 def plain_logits(folder: str, requests: dict, dtype=torch.float64) -> dict:
     raw, weights = read_folder(folder, dtype)
     return {rid: lefisun_plain.forward(raw, weights, toks, dtype) for rid, toks in requests.items()}
+
+
+def rounding_noise(folder: str, requests: dict, dtype, exact: dict) -> dict:
+    """How far rounding alone carries every row: the plain implementation in float32, or in float64 with every
+    tensor a bfloat16 model holds rounded to bfloat16, against the exact rows.  Some rows amplify rounding (a
+    normaliser that nearly cancels, a router between two experts of almost equal score); a row's bound follows it."""
+    raw, weights = read_folder(folder, torch.float64)
+    noise = {}
+    for rid, toks in requests.items():
+        if dtype == torch.float32:
+            noisy = lefisun_plain.forward(raw, weights, toks, torch.float32).double()
+        else:
+            noisy = lefisun_plain.forward(raw, weights, toks, torch.float64, lefisun_plain.to_bfloat16)
+        d = noisy - exact[rid]
+        noise[rid] = (d - d.mean(-1, keepdim=True)).pow(2).mean(-1).sqrt()
+    return noise
+
+
+def compare_with_rounding(collected: dict, exact: dict, noise: dict, *, relative: float, times: float = 4.0,
+                          outliers: float = 0.0) -> float:
+    """Every collected row against the exact one: the root mean square of the difference (its mean taken off) may be
+    `relative` of the exact row's own, or `times` what rounding alone does to that row in the plain implementation,
+    whichever is larger.  A share `outliers` of the rows may lie beyond (bfloat16: the engine's rounding falls
+    otherwise than the plain implementation's, and another expert or key wins).  Returns the worst error in bounds."""
+    errors = {}
+    for (rid, pos) in sorted(collected, key=lambda k: (str(k[0]), k[1])):
+        got, ref = collected[(rid, pos)].double().cpu(), exact[rid][pos].double()
+        assert torch.isfinite(got).all(), f"request {rid!r} position {pos}: logits are not finite"
+        d = got - ref
+        bound = max(relative * max((ref - ref.mean()).pow(2).mean().sqrt().item(), 1e-3), times * float(noise[rid][pos]))
+        errors[(rid, pos)] = (d - d.mean()).pow(2).mean().sqrt().item() / bound
+    beyond = {k: e for k, e in errors.items() if e > 1.0}
+    assert len(beyond) <= outliers * len(errors), (
+        f"{len(beyond)} of {len(errors)} rows beyond the bound; the first: request {next(iter(beyond))[0]!r} position "
+        f"{next(iter(beyond))[1]}: {next(iter(beyond.values())):.2f} x the bound")
+    return max(errors.values())
