@@ -352,8 +352,7 @@ class EmulatedKernels:
         qk[0].copy_((v[:, 0] * q_scale).to(torch.float32))
         qk[1].copy_((v[:, 1] * k_scale).to(torch.float32))
 
-    def memory_gates(self, gates, i_bias, f_bias, qk, state, carried_offset, seg_q_start, seg_q_len, state_slots, steps,
-                     heads, head_dim, cap, den_eps):
+    def memory_gates(self, gates, i_bias, f_bias, state, m_offset, seg_q_start, seg_q_len, state_slots, steps, heads, cap):
         self._count("memory_gates")
         acc = self.acc
         z = gates.to(acc)
@@ -365,44 +364,47 @@ class EmulatedKernels:
         if cap:
             zi, zf = cap * torch.tanh(zi / cap), cap * torch.tanh(zf / cap)
         log_i, log_f = zi, torch.nn.functional.logsigmoid(zf)
-        width = heads * head_dim
         for seg in range(seg_q_start.shape[0]):
             start, length, slot = int(seg_q_start[seg]), int(seg_q_len[seg]), int(state_slots[seg])
-            carried = state[slot, carried_offset:carried_offset + width + heads]
-            nv, m = carried[:width].to(acc).view(heads, head_dim).clone(), carried[width:].to(acc).clone()
+            m = state[slot, m_offset:m_offset + heads].to(acc).clone()
             for t in range(start, start + length):
                 m_new = torch.maximum(log_f[t] + m, log_i[t])
-                a, b = torch.exp(log_f[t] + m - m_new), torch.exp(log_i[t] - m_new)
-                q, k = qk[0, t].to(acc).view(heads, head_dim), qk[1, t].to(acc).view(heads, head_dim)
-                nv = a[:, None] * nv + b[:, None] * k
+                steps[0, t] = torch.exp(log_f[t] + m - m_new).float()
+                steps[1, t] = torch.exp(log_i[t] - m_new).float()
+                steps[2, t] = torch.exp(-m_new).float()
                 m = m_new
-                den = torch.maximum((nv * q).sum(-1).abs(), torch.exp(-m)) + den_eps
-                steps[0, t], steps[1, t], steps[2, t] = a.float(), b.float(), den.float()
-            carried[:width] = nv.reshape(-1).float()
-            carried[width:] = m.float()
+            state[slot, m_offset:m_offset + heads] = m.float()
 
-    def memory_scan(self, qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads, head_dim, value_dim):
+    def memory_scan(self, qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads, head_dim, value_dim,
+                    nq=None, n_offset=0):
         self._count("memory_scan")
         acc = self.acc
-        size = heads * head_dim * value_dim
+        size, width = heads * head_dim * value_dim, heads * head_dim
         for seg in range(seg_q_start.shape[0]):
             start, length, slot = int(seg_q_start[seg]), int(seg_q_len[seg]), int(state_slots[seg])
             S = state[slot, :size].to(acc).view(heads, head_dim, value_dim).clone()
+            nv = state[slot, n_offset:n_offset + width].to(acc).view(heads, head_dim).clone() if steps is not None else None
             for t in range(start, start + length):
                 q, k = qk[0, t].to(acc).view(heads, head_dim), qk[1, t].to(acc).view(heads, head_dim)
                 val = v[t].to(acc).view(heads, value_dim)
                 if steps is not None:
-                    a, b, den = steps[0, t].to(acc), steps[1, t].to(acc), steps[2, t].to(acc)
+                    a, b = steps[0, t].to(acc), steps[1, t].to(acc)
+                    nv = a[:, None] * nv + b[:, None] * k
+                    nq[t] = (nv * q).sum(-1).float()
                 else:
-                    a, b, den = decays.to(acc), torch.ones(heads, dtype=acc), torch.ones(heads, dtype=acc)
+                    a, b = decays.to(acc), torch.ones(heads, dtype=acc)
                 S = a[:, None, None] * S + (b[:, None] * k)[:, :, None] * val[:, None, :]
-                y[t] = (torch.einsum("hdv,hd->hv", S, q) / den[:, None]).reshape(-1).float()
+                y[t] = torch.einsum("hdv,hd->hv", S, q).reshape(-1).float()
             state[slot, :size] = S.reshape(-1).float()
+            if steps is not None:
+                state[slot, n_offset:n_offset + width] = nv.reshape(-1).float()
 
-    def head_norm_gate(self, y, gate, weight, out, heads, eps, activation, scale):
+    def head_norm_gate(self, y, gate, weight, out, heads, eps, activation, scale, nq=None, floor=None, den_eps=0.0):
         self._count("head_norm_gate")
         n, w = y.shape
         v = y.to(self.acc).view(n, heads, w // heads)
+        if nq is not None:
+            v = v / (torch.maximum(nq.to(self.acc).abs(), floor.to(self.acc)) + den_eps)[:, :, None]
         v = (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(n, w)
         if weight is not None:
             v = v * weight.to(self.acc)
@@ -430,10 +432,11 @@ class EmulatedKernels:
             ids[r] = torch.tensor(order, dtype=torch.int32)
             weights[r] = (chosen / (chosen.sum() + eps)).float()
 
-    def moe_plan(self, ids, plan, experts):
+    def moe_plan(self, ids, plan, experts, tile_rows=16):
         self._count("moe_plan")
         flat = ids.reshape(-1).tolist()
         max_tiles = len(flat) // 16 + experts
+        assert tile_rows == 16, "the emulation plans tiles of 16 rows"
         plan.fill_(-7)                       # what the kernels must not read
         tiles = 0
         for e in range(experts):

@@ -158,17 +158,19 @@ def test_a_matrix_memory_whole_and_token_by_token(dtype, kind, heads, d, dv, cap
             positions = torch.arange(start, start + length, dtype=torch.int32, device=DEV)
             ops.memory_inputs(part, positions, None, qk, heads=heads, head_dim=d,
                               q_scale=d ** -0.5 if kind == "exponential" else 1.0, k_scale=1.0 if kind == "exponential" else d ** -0.5)
-            steps = None
+            steps = nq = None
             if kind == "exponential":
                 steps = torch.zeros(3, length, heads, dtype=torch.float32, device=DEV)
-                ops.memory_gates(part[:, 2 * qk_w + 2 * v_w:], w["m.i.b"].float().to(DEV), w["m.f.b"].float().to(DEV), qk, state,
-                                 memory, *seg, steps, heads=heads, head_dim=d, cap=cap, den_eps=1e-6)
+                nq = torch.zeros(length, heads, dtype=torch.float32, device=DEV)
+                ops.memory_gates(part[:, 2 * qk_w + 2 * v_w:], w["m.i.b"].float().to(DEV), w["m.f.b"].float().to(DEV), state,
+                                 memory + qk_w, *seg, steps, heads=heads, cap=cap)
             y = torch.zeros(length, v_w, dtype=torch.float32, device=DEV)
             ops.memory_scan(qk, part[:, 2 * qk_w:2 * qk_w + v_w], steps, decays, state, *seg, y, heads=heads, head_dim=d,
-                            value_dim=dv)
+                            value_dim=dv, nq=nq, n_offset=memory if kind == "exponential" else 0)
             ops.head_norm_gate(y, part[:, 2 * qk_w + v_w:2 * qk_w + 2 * v_w],
                                w["m.norm"].float().to(DEV) if kind == "exponential" else None, out[start:start + length],
-                               heads=heads, eps=eps, activation="sigmoid" if kind == "exponential" else "silu", scale=1.0)
+                               heads=heads, eps=eps, activation="sigmoid" if kind == "exponential" else "silu", scale=1.0,
+                               nq=nq, floor=steps[2] if kind == "exponential" else None, den_eps=1e-6 if kind == "exponential" else 0.0)
         others = [i for i in range(slot_count) if i != slot]
         assert torch.equal(state[others], before[others]), "a state row of another request changed"
         return out, state[slot].clone()
@@ -198,11 +200,12 @@ def test_segments_of_a_batch_keep_their_own_memories(dtype):
         qk = torch.zeros(2, rows.shape[0], qk_w, dtype=torch.float32, device=DEV)
         ops.memory_inputs(rows, pos, None, qk, heads=heads, head_dim=d)
         steps = torch.zeros(3, rows.shape[0], heads, dtype=torch.float32, device=DEV)
-        ops.memory_gates(rows[:, 2 * qk_w + heads * dv:], None, None, qk, st, heads * d * dv, *seg, steps, heads=heads, head_dim=d,
-                         cap=None, den_eps=1e-6)
+        nq = torch.zeros(rows.shape[0], heads, dtype=torch.float32, device=DEV)
+        ops.memory_gates(rows[:, 2 * qk_w + heads * dv:], None, None, st, heads * d * dv + qk_w, *seg, steps, heads=heads, cap=None)
         y = torch.zeros(rows.shape[0], heads * dv, dtype=torch.float32, device=DEV)
-        ops.memory_scan(qk, rows[:, 2 * qk_w:2 * qk_w + heads * dv], steps, None, st, *seg, y, heads=heads, head_dim=d, value_dim=dv)
-        return y
+        ops.memory_scan(qk, rows[:, 2 * qk_w:2 * qk_w + heads * dv], steps, None, st, *seg, y, heads=heads, head_dim=d, value_dim=dv,
+                        nq=nq, n_offset=heads * d * dv)
+        return torch.cat([y, nq, steps[2]], dim=1)
 
     together = run(row, positions, (q_start.to(DEV), q_len.to(DEV), slots.to(DEV)), state)
     for s, (start, length) in enumerate(zip(q_start.tolist(), q_len.tolist())):
@@ -217,7 +220,8 @@ def test_segments_of_a_batch_keep_their_own_memories(dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n,width,ff,count,top,groups,keep", [
     (1, 64, 48, 6, 2, 3, 2), (7, 48, 24, 5, 3, 5, 5), (40, 96, 70, 8, 3, 4, 2), (300, 128, 96, 16, 4, 4, 2), (33, 36, 10, 1, 1, 1, 1),
-    (90, 64, 32, 12, 1, 3, 1), (5, 256, 130, 4, 4, 2, 2), (130, 50, 16, 9, 6, 3, 2)])
+    (90, 64, 32, 12, 1, 3, 1), (5, 256, 130, 4, 4, 2, 2), (130, 50, 16, 9, 6, 3, 2),
+    (300, 128, 192, 4, 2, 2, 1), (700, 64, 64, 3, 1, 1, 1), (450, 192, 128, 6, 3, 3, 2)])     # bfloat16: tiles of 128 rows
 def test_the_router_and_the_experts(dtype, n, width, ff, count, top, groups, keep):
     g = torch.Generator().manual_seed(n + width)
     h = torch.randn(n, width, generator=g).to(dtype)
@@ -246,19 +250,22 @@ def test_the_router_and_the_experts(dtype, n, width, ff, count, top, groups, kee
             order = {e: i for i, e in enumerate(got_ids[r].tolist())}
             for e, a in zip(chosen[r].tolist(), weights[r].tolist()):
                 assert abs(float(wts[r, order[e]]) - a) <= 1e-5 + 1e-4 * a
-    plan = torch.zeros(ops.moe_plan_size(n * top, count), dtype=torch.int32, device=DEV)
-    ops.moe_plan(ids, plan, count)
+    tile = ops.moe_tile_rows(n * top, count, dtype, width, ff)
+    assert tile == (128 if dtype == torch.bfloat16 and (n, ff) in ((300, 192), (700, 64), (450, 128)) else 16)
+    plan = torch.zeros(ops.moe_plan_size(n * top, count, tile), dtype=torch.int32, device=DEV)
+    ops.moe_plan(ids, plan, count, tile)
     tiles = int(plan[0])
-    rows = plan[1 + ops.moe_max_tiles(n * top, count):][:tiles * 16].cpu()
+    rows = plan[1 + ops.moe_max_tiles(n * top, count, tile):][:tiles * tile].cpu()
     assert sorted(a for a in rows.tolist() if a >= 0) == list(range(n * top)), "every assignment has one row"
+    flat_ids = ids.view(-1).cpu()
     for t in range(tiles):
         e = int(plan[1 + t])
-        assert all(int(ids.view(-1)[a]) == e for a in rows[16 * t:16 * t + 16].tolist() if a >= 0)
+        assert all(int(flat_ids[a]) == e for a in rows[tile * t:tile * t + tile].tolist() if a >= 0)
     stack = lambda names: torch.stack([torch.cat([w[f"f.e{e}.{x}"] for x in names]) for e in range(count)]).to(dtype).to(DEV)
     act = torch.zeros(n * top, ff, dtype=dtype, device=DEV)
-    ops.moe_experts_up(x, stack(("gate", "up")), plan, act, top, "silu")
+    ops.moe_experts_up(x, stack(("gate", "up")), plan, act, top, "silu", tile)
     out = torch.full((top, n, width), float("nan"), dtype=torch.float32, device=DEV)
-    ops.moe_experts_down(act, stack(("down",)), plan, wts, out)
+    ops.moe_experts_down(act, stack(("down",)), plan, wts, out, tile)
     rounding = plain.to_bfloat16 if dtype == torch.bfloat16 else plain.same
     want = plain.mixture_of_experts(h.double(), w, "f.", c, rounding)
     got = out.sum(0)

@@ -5,7 +5,10 @@
 //   running maximum m.
 // A fresh request's row is all zeros: S, n and m all start at zero.  Per head and token
 //   S_t = a_t S_(t-1) + b_t k_t v_t^T,    o_t = S_t^T q_t / den_t
-// with (a, b, den) either (the head's fixed decay, 1, 1) or made from the two gates by `memory_gates`.
+// with (a, b) either (the head's fixed decay, 1) and den = 1, or made from the two gates by `memory_gates`; then
+// the normaliser n_t = a_t n_(t-1) + b_t k_t is one more column of the memory (a value that is always 1), the
+// recurrence leaves n_t . q_t beside the columns' sums, and den_t = max(|n_t . q_t|, exp(-m_t)) + eps divides them
+// where the heads are normed (`head_norm_gate`).
 // Everything that enters the recurrence is float32: the rotated queries and keys, the gates, their
 // exponentials, the maximum, the normaliser, the state and every sum.
 #include "common.h"
@@ -62,92 +65,84 @@ WLLM_API int wllm_memory_inputs(const void* row, long long row_stride, const int
 // projections z_i, z_f (a band [n, 2 * heads] of a wider row: the input gates, then the forget gates):
 //   i = cap * tanh((z_i + bias_i) / cap)                 (cap <= 0: no cap)
 //   f = logsigmoid(cap * tanh((z_f + bias_f) / cap))
-//   m_t = max(f + m_(t-1), i);  a = exp(f + m_(t-1) - m_t);  b = exp(i - m_t)
-//   n_t = a n_(t-1) + b k_t;    den = max(|n_t . q_t|, exp(-m_t)) + den_eps
-// steps[0], [1], [2] [n, heads] take a, b and den; n and m are read from and left in the request's row.
-// One wavefront a (head, segment): the chain over the tokens is scalar but for the normaliser, of
-// which a lane keeps every 64th element. ----
-constexpr int kGateRows = 4;          // D <= 64 * kGateRows
-
+//   m_t = max(f + m_(t-1), i);  a = exp(f + m_(t-1) - m_t);  b = exp(i - m_t);  floor = exp(-m_t)
+// steps[0], [1], [2] [n, heads] take a, b and floor; m is read from and left in the request's row (one float a
+// head from `m_offset`).  One wavefront a (head, segment), 64 tokens at a time: a lane bends its token's gates,
+// the chain of maxima (an addition and a maximum a token, the same operations in the same order however the
+// tokens are cut into steps) runs over the 64 in turn with every lane following it, and a lane takes the
+// exponentials of its own token. ----
+__device__ __forceinline__ float from_lane(float v, int lane) {      // `lane` is the same in every lane
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), lane));
+}
 __device__ __forceinline__ float bent(float z, float cap) { return cap > 0.f ? cap * tanhf(z / cap) : z; }
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
 template <typename T>
 __global__ void __launch_bounds__(kWave)
 memory_gates_kernel(const T* __restrict__ gates, long long gates_stride, const float* __restrict__ i_bias,
-                    const float* __restrict__ f_bias, float cap, float den_eps, const float* __restrict__ qk,
-                    float* __restrict__ state, long long state_stride, long long n_offset,
-                    const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
-                    const int* __restrict__ state_slots, float* __restrict__ steps, int tokens, int heads, int d) {
+                    const float* __restrict__ f_bias, float cap, float* __restrict__ state, long long state_stride,
+                    long long m_offset, const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
+                    const int* __restrict__ state_slots, float* __restrict__ steps, int tokens, int heads) {
     const int h = blockIdx.x, seg = blockIdx.y, lane = threadIdx.x;
     const int q_len = seg_q_len[seg], q_start = seg_q_start[seg];
     if (q_len <= 0) return;
-    const size_t width = static_cast<size_t>(heads) * d, all = static_cast<size_t>(tokens) * heads;
-    float* carried = state + static_cast<size_t>(state_slots[seg]) * state_stride + n_offset;
-    float* n_row = carried + static_cast<size_t>(h) * d;
-    float* m_at = carried + width + h;
-    float nv[kGateRows];
-#pragma unroll
-    for (int i = 0; i < kGateRows; ++i) nv[i] = lane + kWave * i < d ? n_row[lane + kWave * i] : 0.f;
+    const size_t all = static_cast<size_t>(tokens) * heads;
+    float* m_at = state + static_cast<size_t>(state_slots[seg]) * state_stride + m_offset + h;
     float m = *m_at;
     const float bi = i_bias ? i_bias[h] : 0.f, bf = f_bias ? f_bias[h] : 0.f;
-    for (int t = 0; t < q_len; ++t) {
-        const size_t token = static_cast<size_t>(q_start + t);
-        const T* g = gates + token * gates_stride;
-        const float li = bent(to_float(g[h]) + bi, cap);
-        const float lf = log_sigmoid(bent(to_float(g[heads + h]) + bf, cap));
-        const float m_new = fmaxf(lf + m, li);
-        const float a = expf(lf + m - m_new), b = expf(li - m_new);
-        const float* q = qk + token * width + static_cast<size_t>(h) * d;
-        const float* k = q + static_cast<size_t>(tokens) * width;
-        float dot = 0.f;
-#pragma unroll
-        for (int i = 0; i < kGateRows; ++i) {
-            const int j = lane + kWave * i;
-            if (j < d) {
-                nv[i] = fmaf(a, nv[i], b * k[j]);
-                dot = fmaf(nv[i], q[j], dot);
-            }
+    for (int t0 = 0; t0 < q_len; t0 += kWave) {
+        const int count = min(kWave, q_len - t0);
+        float li = 0.f, lf = 0.f;
+        if (lane < count) {
+            const T* g = gates + static_cast<size_t>(q_start + t0 + lane) * gates_stride;
+            li = bent(to_float(g[h]) + bi, cap);
+            lf = log_sigmoid(bent(to_float(g[heads + h]) + bf, cap));
         }
-        dot = wave_sum(dot);
-        m = m_new;
-        if (lane == 0) {
-            const size_t at = token * heads + h;
-            steps[at] = a;
-            steps[all + at] = b;
-            steps[2 * all + at] = fmaxf(fabsf(dot), expf(-m_new)) + den_eps;
+        float m_before = 0.f, m_mine = 0.f;
+        for (int t = 0; t < count; ++t) {
+            const float m_new = fmaxf(from_lane(lf, t) + m, from_lane(li, t));
+            if (lane == t) {
+                m_before = m;
+                m_mine = m_new;
+            }
+            m = m_new;
+        }
+        if (lane < count) {
+            const size_t at = static_cast<size_t>(q_start + t0 + lane) * heads + h;
+            steps[at] = expf(lf + m_before - m_mine);
+            steps[all + at] = expf(li - m_mine);
+            steps[2 * all + at] = expf(-m_mine);
         }
     }
-#pragma unroll
-    for (int i = 0; i < kGateRows; ++i)
-        if (lane + kWave * i < d) n_row[lane + kWave * i] = nv[i];
     if (lane == 0) *m_at = m;
 }
 
 WLLM_API int wllm_memory_gates(const void* gates, long long gates_stride, const float* i_bias, const float* f_bias, float cap,
-                               float den_eps, const float* qk, float* state, long long state_stride, long long n_offset,
-                               const int* seg_q_start, const int* seg_q_len, const int* state_slots, float* steps,
-                               int is_bf16, int tokens, int segments, int heads, int d, hipStream_t stream) {
+                               float* state, long long state_stride, long long m_offset, const int* seg_q_start,
+                               const int* seg_q_len, const int* state_slots, float* steps, int is_bf16, int tokens,
+                               int segments, int heads, hipStream_t stream) {
     if (tokens <= 0 || segments <= 0) return 0;
-    if (heads <= 0 || d <= 0 || d > kWave * kGateRows || segments > 65535) return -1;
+    if (heads <= 0 || segments > 65535) return -1;
     const dim3 grid(heads, segments);
     if (is_bf16)
         memory_gates_kernel<bf16><<<grid, kWave, 0, stream>>>(static_cast<const bf16*>(gates), gates_stride, i_bias, f_bias, cap,
-                                                              den_eps, qk, state, state_stride, n_offset, seg_q_start,
-                                                              seg_q_len, state_slots, steps, tokens, heads, d);
+                                                              state, state_stride, m_offset, seg_q_start, seg_q_len,
+                                                              state_slots, steps, tokens, heads);
     else
         memory_gates_kernel<float><<<grid, kWave, 0, stream>>>(static_cast<const float*>(gates), gates_stride, i_bias, f_bias,
-                                                               cap, den_eps, qk, state, state_stride, n_offset, seg_q_start,
-                                                               seg_q_len, state_slots, steps, tokens, heads, d);
+                                                               cap, state, state_stride, m_offset, seg_q_start, seg_q_len,
+                                                               state_slots, steps, tokens, heads);
     return launch_status();
 }
 
 // ---- the recurrence itself.  A workgroup owns (head, segment, 16 columns of P) and walks the segment's
 // tokens in order.  D is cut into 32 slices: a lane is (column, one of four slices), a wavefront four
 // slices, the workgroup's eight wavefronts all of them; a lane keeps its R rows of its column of S in
-// registers.  Tokens are staged 16 at a time through shared memory (q, k, v, a, b, den); a token's o is
+// registers.  Tokens are staged 16 at a time through shared memory (q, k, v, a, b); a token's sum is
 // the slices' partial sums added in a fixed order (within the wavefront, then wavefront by wavefront),
-// so it has the same bits whether the token came alone or inside a prompt. ----
+// so it has the same bits whether the token came alone or inside a prompt.  With `steps` the column behind
+// the last (p = P) is the normaliser: its value is 1 for every token, its rows lie at `n_offset` of the
+// request's row, and its sums go to `nq` [tokens, heads]. ----
 constexpr int kMemTokens = 16;
 constexpr int kMemWaves = 8;
 constexpr int kMemCols = 16;
@@ -156,9 +151,9 @@ constexpr int kMemSlices = kMemWaves * (kWave / kMemCols);
 template <typename T, int R>
 __global__ void __launch_bounds__(kWave * kMemWaves)
 memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long long v_stride, const float* __restrict__ steps,
-                   const float* __restrict__ decays, float* __restrict__ state, long long state_stride,
+                   const float* __restrict__ decays, float* __restrict__ state, long long state_stride, long long n_offset,
                    const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len, const int* __restrict__ state_slots,
-                   float* __restrict__ y, int tokens, int heads, int d, int p_dim) {
+                   float* __restrict__ y, float* __restrict__ nq, int tokens, int heads, int d, int p_dim) {
     extern __shared__ __align__(16) float smem[];
     const int h = blockIdx.x, seg = blockIdx.y, p0 = blockIdx.z * kMemCols;
     const int q_len = seg_q_len[seg], q_start = seg_q_start[seg];
@@ -166,21 +161,24 @@ memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long l
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int col = lane % kMemCols, slice = wave * (kWave / kMemCols) + lane / kMemCols;
     const int p = p0 + col;
-    const bool live = p < p_dim;
+    const bool norm_col = steps != nullptr && p == p_dim;
+    const bool live = p < p_dim || norm_col;
     const int d_pad = (d + 3) / 4 * 4;
     float* q_s = smem;                                   // [kMemTokens][d_pad]
     float* k_s = q_s + kMemTokens * d_pad;               // [kMemTokens][d_pad]
     float* v_s = k_s + kMemTokens * d_pad;               // [kMemTokens][kMemCols]
     float* a_s = v_s + kMemTokens * kMemCols;            // [kMemTokens]
     float* b_s = a_s + kMemTokens;
-    float* den_s = b_s + kMemTokens;
-    float* part_s = den_s + kMemTokens;                  // [kMemTokens][kMemWaves][kMemCols]
+    float* part_s = b_s + kMemTokens;                    // [kMemTokens][kMemWaves][kMemCols]
     const size_t width = static_cast<size_t>(heads) * d, all = static_cast<size_t>(tokens) * heads;
-    float* s_rows = state + static_cast<size_t>(state_slots[seg]) * state_stride + static_cast<size_t>(h) * d * p_dim;
+    float* request = state + static_cast<size_t>(state_slots[seg]) * state_stride;
+    // this lane's column of the state: rows p_dim apart in S, or the normaliser's rows one after the other
+    float* s_rows = norm_col ? request + n_offset + static_cast<size_t>(h) * d : request + static_cast<size_t>(h) * d * p_dim + p;
+    const size_t s_step = norm_col ? 1 : p_dim;
     const int n0 = slice * R;
     float s[R];
 #pragma unroll
-    for (int i = 0; i < R; ++i) s[i] = (live && n0 + i < d) ? s_rows[static_cast<size_t>(n0 + i) * p_dim + p] : 0.f;
+    for (int i = 0; i < R; ++i) s[i] = (live && n0 + i < d) ? s_rows[static_cast<size_t>(n0 + i) * s_step] : 0.f;
     const float fixed = decays ? decays[h] : 1.f;
     for (int t0 = 0; t0 < q_len; t0 += kMemTokens) {
         const int count = min(kMemTokens, q_len - t0);
@@ -195,16 +193,14 @@ memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long l
             const int t = e / kMemCols, c = e % kMemCols;
             v_s[e] = p0 + c < p_dim
                          ? to_float(v[static_cast<size_t>(q_start + t0 + t) * v_stride + static_cast<size_t>(h) * p_dim + p0 + c])
-                         : 0.f;
+                         : (steps != nullptr && p0 + c == p_dim ? 1.f : 0.f);
         }
         if (threadIdx.x < count) {
             const size_t at = static_cast<size_t>(q_start + t0 + threadIdx.x) * heads + h;
             a_s[threadIdx.x] = steps ? steps[at] : fixed;
             b_s[threadIdx.x] = steps ? steps[all + at] : 1.f;
-            den_s[threadIdx.x] = steps ? steps[2 * all + at] : 1.f;
         }
         __syncthreads();
-#pragma unroll 4
         for (int t = 0; t < count; ++t) {
             const float a = a_s[t], bv = b_s[t] * v_s[t * kMemCols + col];
             const float* kt = k_s + t * d_pad + n0;
@@ -223,38 +219,42 @@ memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long l
         __syncthreads();
         for (int e = threadIdx.x; e < count * kMemCols; e += blockDim.x) {
             const int t = e / kMemCols, l = e % kMemCols;
-            if (p0 + l >= p_dim) continue;
+            if (p0 + l > p_dim || (p0 + l == p_dim && steps == nullptr)) continue;
             float total = part_s[(t * kMemWaves) * kMemCols + l];
 #pragma unroll
             for (int w = 1; w < kMemWaves; ++w) total += part_s[(t * kMemWaves + w) * kMemCols + l];
-            y[static_cast<size_t>(q_start + t0 + t) * heads * p_dim + static_cast<size_t>(h) * p_dim + p0 + l] = total / den_s[t];
+            if (p0 + l == p_dim) nq[static_cast<size_t>(q_start + t0 + t) * heads + h] = total;
+            else y[static_cast<size_t>(q_start + t0 + t) * heads * p_dim + static_cast<size_t>(h) * p_dim + p0 + l] = total;
         }
     }
     if (live) {
 #pragma unroll
         for (int i = 0; i < R; ++i)
-            if (n0 + i < d) s_rows[static_cast<size_t>(n0 + i) * p_dim + p] = s[i];
+            if (n0 + i < d) s_rows[static_cast<size_t>(n0 + i) * s_step] = s[i];
     }
 }
 
-// `steps` (float32 [3, tokens, heads]: a, b, den) or, if null, `decays` (float32 [heads]; b = den = 1).
+// `steps` (float32 [3, tokens, heads], of which a and b are read; then `nq` float32 [tokens, heads] takes the
+// normaliser's sums and the normaliser lies at `n_offset` of a request's row) or, if null, `decays` (float32 [heads]; b = 1).
 WLLM_API int wllm_memory_scan(const float* qk, const void* v, long long v_stride, const float* steps, const float* decays,
-                              float* state, long long state_stride, const int* seg_q_start, const int* seg_q_len,
-                              const int* state_slots, float* y, int is_bf16, int tokens, int segments, int heads, int d,
-                              int p_dim, hipStream_t stream) {
+                              float* state, long long state_stride, long long n_offset, const int* seg_q_start,
+                              const int* seg_q_len, const int* state_slots, float* y, float* nq, int is_bf16, int tokens,
+                              int segments, int heads, int d, int p_dim, hipStream_t stream) {
     if (segments <= 0 || tokens <= 0) return 0;
-    if ((!steps) == (!decays)) return -1;
+    if ((!steps) == (!decays) || (steps && !nq)) return -1;
     if (heads <= 0 || d <= 0 || d > 8 * kMemSlices || p_dim <= 0) return -1;
-    if (segments > 65535 || (p_dim + kMemCols - 1) / kMemCols > 65535) return -1;
+    if (segments > 65535 || (p_dim + kMemCols) / kMemCols > 65535) return -1;
     const int r = (d + kMemSlices - 1) / kMemSlices;
     const int d_pad = (d + 3) / 4 * 4;
-    const dim3 grid(heads, segments, (p_dim + kMemCols - 1) / kMemCols);
-    const size_t smem = sizeof(float) * (2 * kMemTokens * d_pad + kMemTokens * kMemCols + 3 * kMemTokens +
+    const int columns = p_dim + (steps ? 1 : 0);
+    const dim3 grid(heads, segments, (columns + kMemCols - 1) / kMemCols);
+    const size_t smem = sizeof(float) * (2 * kMemTokens * d_pad + kMemTokens * kMemCols + 2 * kMemTokens +
                                          kMemTokens * kMemWaves * kMemCols);
 #define LAUNCH(T, R)                                                                                                  \
     memory_scan_kernel<T, R><<<grid, kWave * kMemWaves, smem, stream>>>(qk, static_cast<const T*>(v), v_stride, steps, \
-                                                                        decays, state, state_stride, seg_q_start,    \
-                                                                        seg_q_len, state_slots, y, tokens, heads, d, p_dim)
+                                                                        decays, state, state_stride, n_offset,       \
+                                                                        seg_q_start, seg_q_len, state_slots, y, nq,  \
+                                                                        tokens, heads, d, p_dim)
 #define LAUNCH_R(T)                        \
     if (r <= 1) LAUNCH(T, 1);              \
     else if (r <= 2) LAUNCH(T, 2);         \
@@ -266,40 +266,48 @@ WLLM_API int wllm_memory_scan(const float* qk, const void* v, long long v_stride
     return launch_status();
 }
 
-// ---- out = y / rms_of_the_head(y) * weight * act(gate) * scale: the recurrence's result (float32), every
-// head divided by its own root mean square (eps inside the root), times a weight over the whole row (if
+// ---- out = o / rms_of_the_head(o) * weight * act(gate) * scale with o = y / den: the recurrence's sums (float32),
+// divided by the head's denominator den = max(|nq|, floor) + den_eps if there is one (nq, floor float32 [tokens, heads]),
+// every head divided by its own root mean square (eps inside the root), times a weight over the whole row (if
 // any), times the gate's activation (0: sigmoid, 1: silu) of a band of a wider row; out (the activation
 // type) may be a band too.  One wavefront a (token, head). ----
 template <typename T, int GATE>
 __global__ void __launch_bounds__(kWave)
 head_norm_gate_kernel(const float* __restrict__ y, const T* __restrict__ gate, long long gate_stride,
-                      const float* __restrict__ weight, T* __restrict__ out, long long out_stride, int heads, int p_dim,
+                      const float* __restrict__ weight, T* __restrict__ out, long long out_stride,
+                      const float* __restrict__ nq, const float* __restrict__ floor, float den_eps, int heads, int p_dim,
                       float eps, float scale) {
     const int token = blockIdx.x, h = blockIdx.y;
     const float* yr = y + (static_cast<size_t>(token) * heads + h) * p_dim;
+    const size_t th = static_cast<size_t>(token) * heads + h;
+    const float den = nq ? fmaxf(fabsf(nq[th]), floor[th]) + den_eps : 1.f;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < p_dim; i += kWave) ss = fmaf(yr[i], yr[i], ss);
+    for (int i = threadIdx.x; i < p_dim; i += kWave) {
+        const float o = yr[i] / den;
+        ss = fmaf(o, o, ss);
+    }
     const float inv = 1.f / sqrtf(wave_sum(ss) / static_cast<float>(p_dim) + eps);
     const T* g = gate + static_cast<size_t>(token) * gate_stride + static_cast<size_t>(h) * p_dim;
     T* o = out + static_cast<size_t>(token) * out_stride + static_cast<size_t>(h) * p_dim;
     for (int i = threadIdx.x; i < p_dim; i += kWave) {
         const float z = to_float(g[i]);
         const float sg = 1.f / (1.f + expf(-z));
-        float val = yr[i] * inv;
+        float val = yr[i] / den * inv;
         if (weight) val *= weight[h * p_dim + i];
         o[i] = from_float<T>(val * (GATE == 0 ? sg : z * sg) * scale);
     }
 }
 
 WLLM_API int wllm_head_norm_gate(const float* y, const void* gate, long long gate_stride, const float* weight, void* out,
-                                 long long out_stride, int is_bf16, int gate_kind, int tokens, int heads, int p_dim, float eps,
-                                 float scale, hipStream_t stream) {
+                                 long long out_stride, const float* nq, const float* floor, float den_eps, int is_bf16,
+                                 int gate_kind, int tokens, int heads, int p_dim, float eps, float scale, hipStream_t stream) {
     if (tokens <= 0) return 0;
-    if (heads <= 0 || heads > 65535 || p_dim <= 0 || gate_kind < 0 || gate_kind > 1) return -1;
+    if (heads <= 0 || heads > 65535 || p_dim <= 0 || gate_kind < 0 || gate_kind > 1 || (!nq) != (!floor)) return -1;
     const dim3 grid(tokens, heads);
 #define LAUNCH(T, G)                                                                                                   \
     head_norm_gate_kernel<T, G><<<grid, kWave, 0, stream>>>(y, static_cast<const T*>(gate), gate_stride, weight,       \
-                                                            static_cast<T*>(out), out_stride, heads, p_dim, eps, scale)
+                                                            static_cast<T*>(out), out_stride, nq, floor, den_eps, heads, \
+                                                            p_dim, eps, scale)
     if (is_bf16) { if (gate_kind == 0) LAUNCH(bf16, 0); else LAUNCH(bf16, 1); }
     else { if (gate_kind == 0) LAUNCH(float, 0); else LAUNCH(float, 1); }
 #undef LAUNCH

@@ -5,8 +5,8 @@
 //            `groups` equal groups of neighbours (a group's score: its largest s) may be chosen; the `top`
 //            allowed experts with the largest s are chosen, weights s / (sum of the chosen + eps)
 //   plan     an assignment is a = token * top + slot.  The assignments of one expert lie together, in
-//            tiles of 16 rows (the last tile of an expert padded with -1):
-//            plan[0] = tiles in use; plan[1 + t] = expert of tile t; plan[1 + max_tiles + 16 t + r] = a or -1
+//            tiles of R rows (16 or 128; the last tile of an expert padded with -1):
+//            plan[0] = tiles in use; plan[1 + t] = expert of tile t; plan[1 + max_tiles + R t + r] = a or -1
 //   up       act[a] = activation(x[token] Wg_e^T) * (x[token] Wu_e^T)
 //   down     out[slot][token] = weight[a] * (act[a] Wd_e^T), float32: a stack of `top` partial sums that
 //            whoever adds the feed-forward to the stream adds in order
@@ -21,77 +21,120 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 constexpr int kMoeTile = 16;            // rows of a tile
 constexpr int kMoeMaxExperts = 256;
 
-// ---- the router: one wavefront a token ----
+// ---- the router: one workgroup a token.  The four wavefronts share the experts' dot products (a lane sums its
+// columns in ascending order, the lanes are added in the butterfly's order: the same bits whatever the batch);
+// then the first wavefront, a lane holding the experts lane, lane + 64, ..., takes the softmax, shuts the groups
+// out and picks the top, every choice a maximum over the wavefront and, among equals, the lowest index. ----
+constexpr int kRoutePer = kMoeMaxExperts / kWave;        // experts a lane holds
+
+__device__ __forceinline__ int wave_lowest(int v) { return -static_cast<int>(wave_max(-static_cast<float>(v))); }
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const T* __restrict__ x, const float* __restrict__ router, int* __restrict__ ids, float* __restrict__ weights,
                  int tokens, int width, int experts, int top, int groups, int keep, float eps) {
-    __shared__ float score_s[4][kMoeMaxExperts];
-    __shared__ unsigned char open_s[4][kMoeMaxExperts];
+    __shared__ float z_s[kMoeMaxExperts];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    const int token = blockIdx.x * 4 + wave;
-    if (token >= tokens) return;
+    const int token = blockIdx.x;
     const T* xr = x + static_cast<size_t>(token) * width;
-    float* sc = score_s[wave];
-    unsigned char* open = open_s[wave];
-    for (int e = 0; e < experts; ++e) {
+    for (int e = wave; e < experts; e += 4) {
         const float* w = router + static_cast<size_t>(e) * width;
         float dot = 0.f;
-        for (int c = lane; c < width; c += kWave) dot = fmaf(to_float(xr[c]), w[c], dot);
-        dot = wave_sum(dot);
-        if (lane == 0) sc[e] = dot;
-    }
-    asm volatile("" ::: "memory");
-    if (lane != 0) return;
-    float mx = sc[0];
-    for (int e = 1; e < experts; ++e) mx = fmaxf(mx, sc[e]);
-    float sum = 0.f;
-    for (int e = 0; e < experts; ++e) {
-        sc[e] = expf(sc[e] - mx);
-        sum += sc[e];
-    }
-    for (int e = 0; e < experts; ++e) {
-        sc[e] /= sum;
-        open[e] = 1;
-    }
-    if (keep < groups) {
-        // a group is closed unless it is among the `keep` best: take the best open-able group `keep` times
-        const int per = experts / groups;
-        for (int e = 0; e < experts; ++e) open[e] = 0;
-        for (int pick = 0; pick < keep; ++pick) {
-            int best = -1;
-            float best_score = -1.f;
-            for (int g = 0; g < groups; ++g) {
-                if (open[g * per]) continue;
-                float top_of = sc[g * per];
-                for (int j = 1; j < per; ++j) top_of = fmaxf(top_of, sc[g * per + j]);
-                if (top_of > best_score) {
-                    best_score = top_of;
-                    best = g;
-                }
+        if (width % 4 == 0) {
+#pragma unroll 4
+            for (int c = lane * 4; c < width; c += kWave * 4) {
+                const float4 wv = *reinterpret_cast<const float4*>(w + c);
+                dot = fmaf(to_float(xr[c]), wv.x, dot);
+                dot = fmaf(to_float(xr[c + 1]), wv.y, dot);
+                dot = fmaf(to_float(xr[c + 2]), wv.z, dot);
+                dot = fmaf(to_float(xr[c + 3]), wv.w, dot);
             }
-            for (int j = 0; j < per; ++j) open[best * per + j] = 1;
+        } else {
+            for (int c = lane; c < width; c += kWave) dot = fmaf(to_float(xr[c]), w[c], dot);
         }
+        dot = wave_sum(dot);
+        if (lane == 0) z_s[e] = dot;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    // softmax over all experts
+    float sc[kRoutePer];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < kRoutePer; ++j) {
+        const int e = lane + kWave * j;
+        sc[j] = e < experts ? z_s[e] : -INFINITY;
+        mx = fmaxf(mx, sc[j]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < kRoutePer; ++j) {
+        sc[j] = lane + kWave * j < experts ? expf(sc[j] - mx) : 0.f;
+        sum += sc[j];
+    }
+    sum = wave_sum(sum);
+    // a score that may still be chosen is >= 0; one that may not is -1
+#pragma unroll
+    for (int j = 0; j < kRoutePer; ++j) sc[j] = lane + kWave * j < experts ? sc[j] / sum : -1.f;
+    if (keep < groups) {
+        const int per = experts / groups;
+        float gs[kRoutePer];                     // the scores of the groups lane, lane + 64, ...: their largest member's
+        bool allowed[kRoutePer];
+#pragma unroll
+        for (int j = 0; j < kRoutePer; ++j) {
+            const int g = lane + kWave * j;
+            gs[j] = -1.f;
+            allowed[j] = false;
+            if (g < groups)
+                for (int m = 0; m < per; ++m) gs[j] = fmaxf(gs[j], expf(z_s[g * per + m] - mx) / sum);
+        }
+        for (int pick = 0; pick < keep; ++pick) {
+            float best = -1.f;
+#pragma unroll
+            for (int j = 0; j < kRoutePer; ++j) best = fmaxf(best, gs[j]);
+            best = wave_max(best);
+            int which = kMoeMaxExperts;
+#pragma unroll
+            for (int j = kRoutePer - 1; j >= 0; --j)
+                if (gs[j] == best) which = lane + kWave * j;
+            which = wave_lowest(which);
+#pragma unroll
+            for (int j = 0; j < kRoutePer; ++j) {
+                if (lane + kWave * j == which) gs[j] = -1.f;
+                if ((lane + kWave * j) / per == which) allowed[j] = true;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kRoutePer; ++j)
+            if (!allowed[j]) sc[j] = -1.f;
     }
     float chosen_sum = 0.f;
     int* id = ids + static_cast<size_t>(token) * top;
     float* wt = weights + static_cast<size_t>(token) * top;
     for (int slot = 0; slot < top; ++slot) {
-        int best = -1;
-        float best_score = -1.f;
-        for (int e = 0; e < experts; ++e) {
-            if (open[e] == 1 && sc[e] > best_score) {
-                best_score = sc[e];
-                best = e;
-            }
+        float best = -1.f;
+#pragma unroll
+        for (int j = 0; j < kRoutePer; ++j) best = fmaxf(best, sc[j]);
+        best = wave_max(best);
+        int which = kMoeMaxExperts;
+#pragma unroll
+        for (int j = kRoutePer - 1; j >= 0; --j)
+            if (sc[j] == best) which = lane + kWave * j;
+        which = wave_lowest(which);
+#pragma unroll
+        for (int j = 0; j < kRoutePer; ++j)
+            if (lane + kWave * j == which) sc[j] = -1.f;
+        chosen_sum += best;
+        if (lane == 0) {
+            id[slot] = which;
+            wt[slot] = best;
         }
-        open[best] = 2;
-        id[slot] = best;
-        wt[slot] = best_score;
-        chosen_sum += best_score;
     }
-    const float denom = chosen_sum + eps;
-    for (int slot = 0; slot < top; ++slot) wt[slot] /= denom;
+    if (lane == 0) {
+        const float denom = chosen_sum + eps;
+        for (int slot = 0; slot < top; ++slot) wt[slot] /= denom;
+    }
 }
 
 WLLM_API int wllm_moe_route(const void* x, const float* router, int* ids, float* weights, int is_bf16, int tokens, int width,
@@ -100,21 +143,21 @@ WLLM_API int wllm_moe_route(const void* x, const float* router, int* ids, float*
     if (experts <= 0 || experts > kMoeMaxExperts || groups <= 0 || experts % groups || keep <= 0 || keep > groups || top <= 0 ||
         top > keep * (experts / groups) || width <= 0)
         return -1;
-    const int blocks = (tokens + 3) / 4;
     if (is_bf16)
-        moe_route_kernel<bf16><<<blocks, 256, 0, stream>>>(static_cast<const bf16*>(x), router, ids, weights, tokens, width,
+        moe_route_kernel<bf16><<<tokens, 256, 0, stream>>>(static_cast<const bf16*>(x), router, ids, weights, tokens, width,
                                                            experts, top, groups, keep, eps);
     else
-        moe_route_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<const float*>(x), router, ids, weights, tokens, width,
+        moe_route_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(x), router, ids, weights, tokens, width,
                                                             experts, top, groups, keep, eps);
     return launch_status();
 }
 
-// ---- the plan: one workgroup counts the assignments of every expert, gives each expert its tiles and
-// every assignment a row.  Which row of its expert's tiles an assignment gets depends on the order in
-// which threads arrive; a row's result does not depend on its place. ----
+// ---- the plan: one workgroup counts the assignments of every expert, gives each expert its tiles (of
+// `tile_rows` rows: 16 for the kernels that stream an expert's weights past a few rows, 128 for the kernel that
+// tiles many rows through shared memory) and every assignment a row.  Which row of its expert's tiles an
+// assignment gets depends on the order in which threads arrive; a row's result does not depend on its place. ----
 __global__ void __launch_bounds__(1024)
-moe_plan_kernel(const int* __restrict__ ids, int* __restrict__ plan, int assignments, int experts, int max_tiles) {
+moe_plan_kernel(const int* __restrict__ ids, int* __restrict__ plan, int assignments, int experts, int max_tiles, int tile_rows) {
     __shared__ int count_s[kMoeMaxExperts];
     __shared__ int first_s[kMoeMaxExperts + 1];      // first tile of every expert; [experts]: tiles in use
     int* tile_expert = plan + 1;
@@ -127,7 +170,7 @@ moe_plan_kernel(const int* __restrict__ ids, int* __restrict__ plan, int assignm
         int tiles = 0;
         for (int e = 0; e < experts; ++e) {
             first_s[e] = tiles;
-            tiles += (count_s[e] + kMoeTile - 1) / kMoeTile;
+            tiles += (count_s[e] + tile_rows - 1) / tile_rows;
         }
         first_s[experts] = tiles;
         plan[0] = tiles;
@@ -138,18 +181,19 @@ moe_plan_kernel(const int* __restrict__ ids, int* __restrict__ plan, int assignm
         for (int t = first_s[e]; t < first_s[e + 1]; ++t) tile_expert[t] = e;
         count_s[e] = 0;                              // from here on: rows of the expert already given out
     }
-    for (int i = threadIdx.x; i < tiles * kMoeTile; i += blockDim.x) rows[i] = -1;
+    for (int i = threadIdx.x; i < tiles * tile_rows; i += blockDim.x) rows[i] = -1;
     __syncthreads();
     for (int a = threadIdx.x; a < assignments; a += blockDim.x) {
         const int e = ids[a];
-        rows[first_s[e] * kMoeTile + atomicAdd(&count_s[e], 1)] = a;
+        rows[first_s[e] * tile_rows + atomicAdd(&count_s[e], 1)] = a;
     }
 }
 
-WLLM_API int wllm_moe_plan(const int* ids, int* plan, int assignments, int experts, int max_tiles, hipStream_t stream) {
+WLLM_API int wllm_moe_plan(const int* ids, int* plan, int assignments, int experts, int max_tiles, int tile_rows,
+                           hipStream_t stream) {
     if (assignments <= 0) return 0;
-    if (experts <= 0 || experts > kMoeMaxExperts || max_tiles < assignments / kMoeTile + experts) return -1;
-    moe_plan_kernel<<<1, 1024, 0, stream>>>(ids, plan, assignments, experts, max_tiles);
+    if (experts <= 0 || experts > kMoeMaxExperts || tile_rows <= 0 || max_tiles < assignments / tile_rows + experts) return -1;
+    moe_plan_kernel<<<1, 1024, 0, stream>>>(ids, plan, assignments, experts, max_tiles, tile_rows);
     return launch_status();
 }
 
@@ -174,6 +218,12 @@ template <> struct MoeFrag<bf16> {
         }
         v = t.v;
     }
+    template <bool STREAM = false>
+    __device__ __forceinline__ void whole(const bf16* p) {           // 8 keys that are all there, 16-byte aligned
+        union { uint4 u; bf16x8_t v; } t;
+        t.u = STREAM ? load_streamed(p) : *reinterpret_cast<const uint4*>(p);
+        v = t.v;
+    }
     static __device__ __forceinline__ float4_t mma(const MoeFrag& a, const MoeFrag& b, float4_t acc) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
     }
@@ -193,6 +243,11 @@ template <> struct MoeFrag<float> {
                 for (int j = 0; j < 4; ++j) v[j] = k + j < K ? p[k + j] : 0.f;
             }
         }
+    }
+    template <bool STREAM = false>
+    __device__ __forceinline__ void whole(const float* p) {
+        const float4 t = *reinterpret_cast<const float4*>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
     }
     static __device__ __forceinline__ float4_t mma(const MoeFrag& a, const MoeFrag& b, float4_t acc) {
 #pragma unroll
@@ -222,14 +277,33 @@ moe_up_kernel(const T* __restrict__ x, const T* __restrict__ w, const int* __res
     const T* wu = wg + static_cast<size_t>(ff) * K;
     float4_t acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
     constexpr int kChunk = MoeFrag<T>::kChunk, kPer = MoeFrag<T>::kPer;
-    for (int k0 = 0; k0 < K; k0 += kChunk) {
-        MoeFrag<T> fx, fg, fu;
-        const int k = k0 + g * kPer;
-        fx.load(xr, k, K, a_i >= 0);
-        fg.load(wg, k, K, w_live);
-        fu.load(wu, k, K, w_live);
-        acc_g = MoeFrag<T>::mma(fg, fx, acc_g);
-        acc_u = MoeFrag<T>::mma(fu, fx, acc_u);
+    if (K % (4 * kChunk) == 0) {
+        // every fragment is whole (rows that stand for nothing read row 0, and their sums are dropped); four
+        // chunks' loads are asked for before the first product
+        for (int k0 = g * kPer; k0 < K; k0 += 4 * kChunk) {
+            MoeFrag<T> fx[4], fg[4], fu[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                fx[u].whole(xr + k0 + u * kChunk);
+                fg[u].template whole<true>(wg + k0 + u * kChunk);
+                fu[u].template whole<true>(wu + k0 + u * kChunk);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                acc_g = MoeFrag<T>::mma(fg[u], fx[u], acc_g);
+                acc_u = MoeFrag<T>::mma(fu[u], fx[u], acc_u);
+            }
+        }
+    } else {
+        for (int k0 = 0; k0 < K; k0 += kChunk) {
+            MoeFrag<T> fx, fg, fu;
+            const int k = k0 + g * kPer;
+            fx.load(xr, k, K, a_i >= 0);
+            fg.load(wg, k, K, w_live);
+            fu.load(wu, k, K, w_live);
+            acc_g = MoeFrag<T>::mma(fg, fx, acc_g);
+            acc_u = MoeFrag<T>::mma(fu, fx, acc_u);
+        }
     }
     if (a_i < 0) return;
     T* out = act + static_cast<size_t>(a_i) * ff;
@@ -273,12 +347,25 @@ moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w, const int* _
     const T* wd = w + (static_cast<size_t>(e) * width + (w_live ? c0 + i : 0)) * ff;
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
     constexpr int kChunk = MoeFrag<T>::kChunk, kPer = MoeFrag<T>::kPer;
-    for (int k0 = 0; k0 < ff; k0 += kChunk) {
-        MoeFrag<T> fx, fw;
-        const int k = k0 + g * kPer;
-        fx.load(xr, k, ff, a_i >= 0);
-        fw.load(wd, k, ff, w_live);
-        acc = MoeFrag<T>::mma(fw, fx, acc);
+    if (ff % (4 * kChunk) == 0) {
+        for (int k0 = g * kPer; k0 < ff; k0 += 4 * kChunk) {
+            MoeFrag<T> fx[4], fw[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                fx[u].whole(xr + k0 + u * kChunk);
+                fw[u].template whole<true>(wd + k0 + u * kChunk);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc = MoeFrag<T>::mma(fw[u], fx[u], acc);
+        }
+    } else {
+        for (int k0 = 0; k0 < ff; k0 += kChunk) {
+            MoeFrag<T> fx, fw;
+            const int k = k0 + g * kPer;
+            fx.load(xr, k, ff, a_i >= 0);
+            fw.load(wd, k, ff, w_live);
+            acc = MoeFrag<T>::mma(fw, fx, acc);
+        }
     }
     if (a_i < 0) return;
     const float weight = weights[a_i];
@@ -301,5 +388,178 @@ WLLM_API int wllm_moe_down(const void* act, const void* w, const int* plan, int 
     else
         moe_down_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(act), static_cast<const float*>(w), plan,
                                                          max_tiles, weights, out, tokens, ff, width, top);
+    return launch_status();
+}
+
+// ---- many rows an expert: the two products in tiles of 128 rows of one expert by 128 rows of its weights,
+// through shared memory, as the framework's tiled product does it (four wavefronts of 64 x 64, stages of 64 keys
+// that go from memory straight into shared memory in an XOR-swizzled order, two stages in turn, two workgroups a
+// compute unit).  What differs: a tile's rows of x are gathered (row r of tile t is the assignment the plan names:
+// the token's row of x for the first product, the assignment's row of act for the second), the weights are the
+// tile's expert's, and a row's result goes where its assignment belongs.  A row's sums run over k in ascending
+// stages whatever tile it lies in.  Workgroups that share an expert's rows of w lie 8 indices apart, on one XCD.
+// bfloat16; K a multiple of 64. ----
+constexpr int kBigRows = 128;
+constexpr int kBigKeys = 64;
+constexpr int kBigRowBytes = kBigKeys * 2;
+constexpr int kBigStageBytes = 2 * kBigRows * kBigRowBytes;
+
+union MoeTFrag {
+    uint4 u;
+    bf16x8_t v;
+};
+
+// 16 bytes a lane from base + offset into shared memory at dst + 16 * lane (M0 is put back as it was).
+static __device__ __forceinline__ void moe_load_to_shared(const void* base, uint32_t offset, void* dst) {
+    const uint32_t lds_address = __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)dst)));
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0) : "v"(offset), "s"(base), "s"(lds_address) : "memory");
+}
+
+// GATED: 0 the second product (out32[a % top][a / top][n] = weight[a] * sum), 1 + the activation's number the
+// first (act[a][n] = activation(gate) * up; w holds an expert's N gate rows, then its N up rows).
+template <int GATED>
+__global__ void __launch_bounds__(256, 2)
+moe_tile_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const int* __restrict__ plan, int max_tiles,
+                bf16* __restrict__ act, float* __restrict__ out32, const float* __restrict__ weights, int N, int K, int top,
+                int tokens) {
+    constexpr int kWaves = 4, kStages = 2;
+    constexpr int kWBytes = kBigRows * kBigRowBytes;
+    constexpr int kLoads = 2 * kBigRows / 8 / kWaves;
+    extern __shared__ __align__(16) unsigned char tiles_s[];
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int i = lane % 16, g = lane / 16;
+    const int wm = wave / 2, wn = wave % 2;
+    const int xcd = blockIdx.x % 8, j = blockIdx.x / 8;
+    const int m_tile = j % max_tiles;
+    const int n_tile = (j / max_tiles) * 8 + xcd;
+    constexpr int kColumns = GATED ? kBigRows / 2 : kBigRows;
+    const int n_base = n_tile * kColumns;
+    if (m_tile >= plan[0] || n_base >= N) return;
+    const int e = plan[1 + m_tile];
+    const int* rows = plan + 1 + max_tiles + m_tile * kBigRows;
+    const int stages = K / kBigKeys;
+    const bf16* we = w + static_cast<size_t>(e) * (GATED ? 2 : 1) * N * K;
+
+    const int chunk = (lane % 8) ^ (lane / 8);
+    uint32_t offset[kLoads];
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+        const int r = 8 * (wave + kWaves * u) + lane / 8;
+        size_t row;
+        if (r < kBigRows) {
+            if (GATED) row = r < 64 ? min(n_base + r, N - 1) : N + min(n_base + r - 64, N - 1);
+            else row = min(n_base + r, N - 1);
+        } else {
+            const int a = rows[r - kBigRows];
+            row = a < 0 ? 0 : (GATED ? a / top : a);
+        }
+        offset[u] = static_cast<uint32_t>((row * K + chunk * 8) * 2);
+    }
+    const unsigned char* w_bytes = reinterpret_cast<const unsigned char*>(we);
+    const unsigned char* x_bytes = reinterpret_cast<const unsigned char*>(x);
+    auto issue = [&](int stage, int s) {
+        const unsigned char* wb = w_bytes + static_cast<size_t>(s) * kBigRowBytes;
+        const unsigned char* xb = x_bytes + static_cast<size_t>(s) * kBigRowBytes;
+#pragma unroll
+        for (int u = 0; u < kLoads; ++u) {
+            const int q = wave + kWaves * u;
+            moe_load_to_shared(q < kBigRows / 8 ? wb : xb, offset[u], tiles_s + stage * kBigStageBytes + q * 1024);
+        }
+    };
+
+    float4_t acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+    int w_row_s[4], x_row_s[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        w_row_s[a] = GATED ? (a < 2 ? wn * 32 + 16 * a + i : 64 + wn * 32 + 16 * (a - 2) + i) : wn * 64 + 16 * a + i;
+        x_row_s[a] = wm * 64 + 16 * a + i;
+    }
+    issue(0, 0);
+    for (int s = 0; s < stages; ++s) {
+        const int stage = s % kStages;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (s + 1 < stages) issue((s + 1) % kStages, s + 1);
+        const unsigned char* ws = tiles_s + stage * kBigStageBytes;
+        const unsigned char* xs = ws + kWBytes;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int place = ((ks * 4 + g) ^ (i % 8)) * 16;
+            MoeTFrag fw[4], fx[4];
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                fw[a].u = *reinterpret_cast<const uint4*>(ws + w_row_s[a] * 128 + place);
+                fx[a].u = *reinterpret_cast<const uint4*>(xs + x_row_s[a] * 128 + place);
+            }
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[a].v, fx[b].v, acc[a][b], 0, 0, 0);
+        }
+    }
+
+    // lane (i, g) holds, of tile (a, b), the tile's row 16 b + i and columns 4g .. 4g + 3 of the tile's 16
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const int asg = rows[wm * 64 + 16 * b + i];
+        if (asg < 0) continue;
+        if (GATED) {
+            bf16* o_row = act + static_cast<size_t>(asg) * N;
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                const int n = n_base + wn * 32 + 16 * a + 4 * g;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (n + v < N)
+                        o_row[n + v] = from_float<bf16>(activate<(GATED > 0 ? GATED - 1 : 0)>(acc[a][b][v]) * acc[a + 2][b][v]);
+            }
+        } else {
+            const float weight = weights[asg];
+            float* o_row = out32 + (static_cast<size_t>(asg % top) * tokens + asg / top) * N;
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const int n = n_base + wn * 64 + 16 * a + 4 * g;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (n + v < N) o_row[n + v] = weight * acc[a][b][v];
+            }
+        }
+    }
+}
+
+// The first product (activation >= 0: `act` [assignments, N] from x [tokens, K] and w [experts, 2N, K]) or the second
+// (activation < 0: out32 [top, tokens, N] from x = act [assignments, K] and w [experts, N, K]) over a plan of tiles of
+// 128 rows.  Returns -1 for sizes it does not take (K no multiple of 64, operands of 4 GiB).
+WLLM_API int wllm_moe_tiles(const void* x, const void* w, const int* plan, int max_tiles, void* act, float* out32,
+                            const float* weights, int activation, int x_rows, int N, int K, int top, int tokens,
+                            hipStream_t stream) {
+    if (max_tiles <= 0 || x_rows <= 0) return 0;
+    if (N <= 0 || K < kBigKeys || K % kBigKeys || top <= 0 || tokens <= 0 || activation >= kActivations) return -1;
+    const bool gated = activation >= 0;
+    if ((gated && !act) || (!gated && (!out32 || !weights))) return -1;
+    if (static_cast<size_t>(gated ? 2 : 1) * N * K * 2 >= (size_t(1) << 32) || static_cast<size_t>(x_rows) * K * 2 >= (size_t(1) << 32))
+        return -1;
+    const int columns = gated ? kBigRows / 2 : kBigRows;
+    const int n_tiles = (N + columns - 1) / columns;
+    const long long blocks = static_cast<long long>((n_tiles + 7) / 8 * 8) * max_tiles;
+    if (blocks > 0x7fffffffLL) return -1;
+    const dim3 grid(static_cast<unsigned>(blocks));
+    const bf16* xp = static_cast<const bf16*>(x);
+    const bf16* wp = static_cast<const bf16*>(w);
+#define LAUNCH(GATED)                                                                                                 \
+    moe_tile_kernel<GATED><<<grid, 256, 2 * kBigStageBytes, stream>>>(xp, wp, plan, max_tiles, static_cast<bf16*>(act), \
+                                                                      out32, weights, N, K, top, tokens)
+    if (!gated) { LAUNCH(0); }
+    else { WLLM_BY_ACTIVATION(activation, LAUNCH(ACT + 1)) }
+#undef LAUNCH
     return launch_status();
 }

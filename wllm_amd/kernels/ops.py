@@ -918,68 +918,71 @@ def memory_inputs(row: torch.Tensor, positions: torch.Tensor, inv_freq: Optional
         call("memory_inputs", row, positions, inv_freq, qk, heads, head_dim, float(q_scale), float(k_scale))
 
 
-def memory_gates(gates: torch.Tensor, i_bias: Optional[torch.Tensor], f_bias: Optional[torch.Tensor], qk: torch.Tensor,
-                 state: torch.Tensor, carried_offset: int, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
-                 state_slots: torch.Tensor, steps: torch.Tensor, *, heads: int, head_dim: int,
-                 cap: Optional[float] = None, den_eps: float = 1e-6) -> None:
+def memory_gates(gates: torch.Tensor, i_bias: Optional[torch.Tensor], f_bias: Optional[torch.Tensor], state: torch.Tensor,
+                 m_offset: int, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor,
+                 steps: torch.Tensor, *, heads: int, cap: Optional[float] = None) -> None:
     """Exponential gates held in range by a running maximum, over each segment's tokens in order.  Per head:
         i = cap tanh((z_i + i_bias) / cap);  f = logsigmoid(cap tanh((z_f + f_bias) / cap))   (cap None: no cap)
-        m_t = max(f + m_(t-1), i);  a = exp(f + m_(t-1) - m_t);  b = exp(i - m_t)
-        n_t = a n_(t-1) + b k_t;    den = max(|n_t . q_t|, exp(-m_t)) + den_eps
+        m_t = max(f + m_(t-1), i);  a = exp(f + m_(t-1) - m_t);  b = exp(i - m_t);  floor = exp(-m_t)
     gates T [n, 2 * heads] (may be a band): z_i of all heads, then z_f; biases float32 [heads] or None;
-    qk float32 [2, n, heads * head_dim] as `memory_inputs` left it; state float32 [slots, W] holds, from
-    column `carried_offset` of row state_slots[segment], n as [heads, head_dim] and then m as [heads]
-    (zeros for a fresh request); steps float32 [3, n, heads] takes a, b and den.  All float32."""
+    state float32 [slots, W] holds m as [heads] from column `m_offset` of row state_slots[segment]
+    (zeros for a fresh request); steps float32 [3, n, heads] takes a, b and floor.  All float32."""
     _need(gates.dim() == 2 and gates.dtype in _ACT, "gates: expected T [n, 2 * heads]")
     n = gates.shape[0]
     _band(gates, "gates", gates.dtype, n, 2 * heads)
-    _need(0 < head_dim <= 256, "head_dim: from 1 to 256")
     for t, name in ((i_bias, "i_bias"), (f_bias, "f_bias")):
         if t is not None:
             _dense(t, name, torch.float32, (heads,))
-    _dense(qk, "qk", torch.float32, (2, n, heads * head_dim))
     _dense(state, "state", torch.float32)
-    _need(state.dim() == 2 and 0 <= carried_offset and carried_offset + heads * head_dim + heads <= state.shape[1],
-          "state: a row holds n and m from carried_offset")
+    _need(state.dim() == 2 and 0 <= m_offset and m_offset + heads <= state.shape[1], "state: a row holds m from m_offset")
     _segments(seg_q_start, seg_q_len, state_slots)
     _dense(steps, "steps", torch.float32, (3, n, heads))
     _need(cap is None or cap > 0, "cap must be positive or None")
     if n:
-        call("memory_gates", gates, i_bias, f_bias, qk, state, int(carried_offset), seg_q_start, seg_q_len, state_slots,
-             steps, heads, head_dim, cap, float(den_eps))
+        call("memory_gates", gates, i_bias, f_bias, state, int(m_offset), seg_q_start, seg_q_len, state_slots, steps, heads, cap)
 
 
 def memory_scan(qk: torch.Tensor, v: torch.Tensor, steps: Optional[torch.Tensor], decays: Optional[torch.Tensor],
                 state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor,
-                y: torch.Tensor, *, heads: int, head_dim: int, value_dim: int) -> None:
+                y: torch.Tensor, *, heads: int, head_dim: int, value_dim: int, nq: Optional[torch.Tensor] = None,
+                n_offset: int = 0) -> None:
     """The matrix memory's recurrence over each segment's tokens in order, from and into the request's
-    carried state.  Per head:  S = a S + b k v^T;  y = S^T q / den  with (a, b, den) of the token from
-    `steps` (float32 [3, n, heads]) or, with `decays` (float32 [heads]) instead, (decays[h], 1, 1).
-    qk float32 [2, n, heads * head_dim]: queries, then keys; v T [n, heads * value_dim] (may be a band);
-    state float32 [slots, W], whose row state_slots[segment] begins with S as [heads, head_dim, value_dim];
-    y float32 [n, heads * value_dim].  All of the recurrence is float32."""
+    carried state.  Per head:  S = a S + b k v^T;  y = S^T q  with (a, b) of the token from `steps` (float32
+    [3, n, heads], of which the first two are read) or, with `decays` (float32 [heads]) instead, (decays[h], 1).
+    With `steps` the normaliser n = a n + b k is carried too, as [heads, head_dim] from column `n_offset` of the
+    request's row, and nq (float32 [n, heads]) takes n . q.  qk float32 [2, n, heads * head_dim]: queries, then
+    keys; v T [n, heads * value_dim] (may be a band); state float32 [slots, W], whose row state_slots[segment]
+    begins with S as [heads, head_dim, value_dim]; y float32 [n, heads * value_dim].  All of the recurrence is float32."""
     _need((steps is None) != (decays is None), "steps or decays, one of the two")
     _need(v.dim() == 2 and v.dtype in _ACT, "v: expected T [n, heads * value_dim]")
     n = v.shape[0]
     _band(v, "v", v.dtype, n, heads * value_dim)
     _need(0 < head_dim <= 256 and value_dim > 0, "head_dim: from 1 to 256")
     _dense(qk, "qk", torch.float32, (2, n, heads * head_dim))
+    _dense(state, "state", torch.float32)
+    memory = heads * head_dim * value_dim
+    _need(state.dim() == 2 and state.shape[1] >= memory, "state: a row holds at least [heads, D, P]")
     if steps is not None:
         _dense(steps, "steps", torch.float32, (3, n, heads))
+        _need(nq is not None, "nq: the normaliser's sums go with steps")
+        _dense(nq, "nq", torch.float32, (n, heads))
+        _need(memory <= n_offset and n_offset + heads * head_dim <= state.shape[1], "state: the normaliser lies behind S")
     else:
         _dense(decays, "decays", torch.float32, (heads,))
-    _dense(state, "state", torch.float32)
-    _need(state.dim() == 2 and state.shape[1] >= heads * head_dim * value_dim, "state: a row holds at least [heads, D, P]")
+        _need(nq is None, "nq: only with steps")
     _segments(seg_q_start, seg_q_len, state_slots)
     _dense(y, "y", torch.float32, (n, heads * value_dim))
     if n:
-        call("memory_scan", qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads, head_dim, value_dim)
+        call("memory_scan", qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads, head_dim, value_dim, nq,
+             int(n_offset))
 
 
 def head_norm_gate(y: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], out: torch.Tensor, *, heads: int,
-                   eps: float, activation: str = "sigmoid", scale: float = 1.0) -> None:
-    """out = y / rms_of_its_head(y) * weight * act(gate) * scale: every one of `heads` equal parts of a row
-    of y is divided by sqrt(mean of its squares + eps).  y float32 [n, W]; gate T [n, W] and out T [n, W]
+                   eps: float, activation: str = "sigmoid", scale: float = 1.0, nq: Optional[torch.Tensor] = None,
+                   floor: Optional[torch.Tensor] = None, den_eps: float = 0.0) -> None:
+    """out = o / rms_of_its_head(o) * weight * act(gate) * scale with o = y / den: every one of `heads` equal parts
+    of a row of y is divided by its denominator den = max(|nq|, floor) + den_eps (nq, floor float32 [n, heads]; without
+    them den = 1) and then by sqrt(mean of its squares + eps).  y float32 [n, W]; gate T [n, W] and out T [n, W]
     may be bands of wider tensors; weight float32 [W] or None; activation "sigmoid" or "silu"."""
     _need(activation in GATE_KINDS, lambda: f"activation {activation!r}: expected one of {sorted(GATE_KINDS)}")
     _dense(y, "y", torch.float32)
@@ -990,25 +993,37 @@ def head_norm_gate(y: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.T
     _band(out, "out", gate.dtype, n, w)
     if weight is not None:
         _dense(weight, "weight", torch.float32, (w,))
+    _need((nq is None) == (floor is None), "nq and floor go together")
+    if nq is not None:
+        _dense(nq, "nq", torch.float32, (n, heads))
+        _dense(floor, "floor", torch.float32, (n, heads))
     if n:
-        call("head_norm_gate", y, gate, weight, out, heads, float(eps), activation, float(scale))
+        call("head_norm_gate", y, gate, weight, out, heads, float(eps), activation, float(scale), nq, floor, float(den_eps))
 
 
 # ---- a mixture of experts ------------------------------------------------------------------------------
-MOE_TILE_ROWS = 16
+MOE_TILE_ROWS = 16           # rows of a tile of the kernels that stream an expert's weights past a few rows
+MOE_BIG_TILE_ROWS = 128      # rows of a tile of the kernel that tiles many rows an expert through shared memory
 MOE_MAX_EXPERTS = 256
 
 
-def moe_max_tiles(assignments: int, experts: int) -> int:
-    """The most tiles of `MOE_TILE_ROWS` rows that `assignments` (token, expert) pairs can fill when the
+def moe_tile_rows(assignments: int, experts: int, dtype, *inner_sizes: int) -> int:
+    """The tile a step's plan should have: tiles of 128 rows where the experts get some tens of rows each on average
+    (a prompt's portion) and the tiled kernel takes the sizes (bfloat16, inner sizes in multiples of 64), else 16."""
+    big = dtype == torch.bfloat16 and assignments >= 32 * experts and all(k % 64 == 0 and k >= 64 for k in inner_sizes)
+    return MOE_BIG_TILE_ROWS if big else MOE_TILE_ROWS
+
+
+def moe_max_tiles(assignments: int, experts: int, tile_rows: int = MOE_TILE_ROWS) -> int:
+    """The most tiles of `tile_rows` rows that `assignments` (token, expert) pairs can fill when the
     pairs of an expert lie together and every expert's last tile may be partly empty."""
-    return assignments // MOE_TILE_ROWS + experts
+    return assignments // tile_rows + experts
 
 
-def moe_plan_size(assignments: int, experts: int) -> int:
+def moe_plan_size(assignments: int, experts: int, tile_rows: int = MOE_TILE_ROWS) -> int:
     """int32 elements of the plan `moe_plan` writes: the number of tiles in use, a tile's expert for
     every tile there is room for, and the rows of every tile."""
-    return 1 + moe_max_tiles(assignments, experts) * (1 + MOE_TILE_ROWS)
+    return 1 + moe_max_tiles(assignments, experts, tile_rows) * (1 + tile_rows)
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, *, groups: int = 1,
@@ -1035,24 +1050,34 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, ids: torch.Tensor, weights:
         call("moe_route", x, router, ids, weights, int(groups), int(keep), float(eps))
 
 
-def moe_plan(ids: torch.Tensor, plan: torch.Tensor, experts: int) -> None:
+def moe_plan(ids: torch.Tensor, plan: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS) -> None:
     """Sorts a step's assignments (a = token * top + slot, expert ids.flat[a]) by expert, in tiles of
-    `MOE_TILE_ROWS` rows: plan[0] = tiles in use; plan[1 + t] = expert of tile t; plan[1 + T + 16 t + r] =
-    the assignment in row r of tile t, or -1, with T = moe_max_tiles(ids.numel(), experts).  An expert's
+    `tile_rows` rows (R): plan[0] = tiles in use; plan[1 + t] = expert of tile t; plan[1 + T + R t + r] =
+    the assignment in row r of tile t, or -1, with T = moe_max_tiles(ids.numel(), experts, R).  An expert's
     assignments lie together in any order.  ids int32 [n, top]; plan int32 [moe_plan_size(...)]."""
     _dense(ids, "ids", torch.int32)
     _need(ids.dim() == 2, "ids: expected [n, top]")
     _need(0 < experts <= MOE_MAX_EXPERTS, f"experts: from 1 to {MOE_MAX_EXPERTS}")
-    _dense(plan, "plan", torch.int32, (moe_plan_size(ids.numel(), experts),))
+    _need(tile_rows in (MOE_TILE_ROWS, MOE_BIG_TILE_ROWS), "tile_rows: 16 or 128")
+    _dense(plan, "plan", torch.int32, (moe_plan_size(ids.numel(), experts, tile_rows),))
     if ids.numel():
-        call("moe_plan", ids, plan, int(experts))
+        call("moe_plan", ids, plan, int(experts), int(tile_rows))
+
+
+def _big_tiles(tile_rows: int, dtype, inner: int) -> bool:
+    _need(tile_rows in (MOE_TILE_ROWS, MOE_BIG_TILE_ROWS), "tile_rows: 16 or 128")
+    if tile_rows == MOE_BIG_TILE_ROWS:
+        _need(dtype == torch.bfloat16 and inner % 64 == 0 and inner >= 64,
+              "tiles of 128 rows: bfloat16 and an inner size that is a multiple of 64")
+        return True
+    return False
 
 
 def moe_experts_up(x: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, act: torch.Tensor, top: int,
-                   activation: str) -> None:
-    """act[a] = activation(x[a // top] Wg_e^T) * (x[a // top] Wu_e^T) for every assignment a of the plan, e
-    its expert.  x T [n, width]; w T [experts, 2 * ff, width]: an expert's gate rows, then its up rows; act
-    T [n * top, ff]; float32 sums."""
+                   activation: str, tile_rows: int = MOE_TILE_ROWS) -> None:
+    """act[a] = activation(x[a // top] Wg_e^T) * (x[a // top] Wu_e^T) for every assignment a of the plan (of tiles of
+    `tile_rows` rows), e its expert.  x T [n, width]; w T [experts, 2 * ff, width]: an expert's gate rows, then its
+    up rows; act T [n * top, ff]; float32 sums."""
     _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {sorted(ACTIVATIONS)}")
     _dense(x, "x", _ACT)
     _need(x.dim() == 2, "x: expected [n, width]")
@@ -1061,13 +1086,16 @@ def moe_experts_up(x: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, act: to
     _need(w.dim() == 3 and w.shape[2] == width and w.shape[1] % 2 == 0, "w: expected [experts, 2 * ff, width]")
     experts, ff = w.shape[0], w.shape[1] // 2
     _dense(act, "act", x.dtype, (n * top, ff))
-    _dense(plan, "plan", torch.int32, (moe_plan_size(n * top, experts),))
+    _dense(plan, "plan", torch.int32, (moe_plan_size(n * top, experts, tile_rows),))
     if n:
-        call("moe_experts_up", x, w, plan, act, int(top), activation)
+        if _big_tiles(tile_rows, x.dtype, width):
+            call("moe_experts_up_tiled", x, w, plan, act, int(top), activation)
+        else:
+            call("moe_experts_up", x, w, plan, act, int(top), activation)
 
 
 def moe_experts_down(act: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, weights: torch.Tensor,
-                     out: torch.Tensor) -> None:
+                     out: torch.Tensor, tile_rows: int = MOE_TILE_ROWS) -> None:
     """out[a % top][a // top] = weights.flat[a] * (act[a] Wd_e^T) for every assignment a of the plan: the
     experts' weighted results as a stack of `top` float32 partial sums over the tokens.  act T [n * top, ff];
     w T [experts, width, ff]; weights float32 [n, top]; out float32 [top, n, width]."""
@@ -1079,9 +1107,12 @@ def moe_experts_down(act: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, wei
     _dense(w, "w", act.dtype)
     _need(w.dim() == 3 and w.shape[2] == act.shape[1], "w: expected [experts, width, ff]")
     _dense(out, "out", torch.float32, (top, n, w.shape[1]))
-    _dense(plan, "plan", torch.int32, (moe_plan_size(n * top, w.shape[0]),))
+    _dense(plan, "plan", torch.int32, (moe_plan_size(n * top, w.shape[0], tile_rows),))
     if n:
-        call("moe_experts_down", act, w, plan, weights, out)
+        if _big_tiles(tile_rows, act.dtype, act.shape[1]):
+            call("moe_experts_down_tiled", act, w, plan, weights, out)
+        else:
+            call("moe_experts_down", act, w, plan, weights, out)
 
 
 # ---- the framework's own operations that go through the same door as a part's ------------------
@@ -1211,35 +1242,37 @@ def _register_own() -> None:
                     p(row), row.stride(0), p(positions), p(inv_freq), p(qk), bf(row), row.shape[0], heads, head_dim,
                     2 * inv_freq.shape[0] if inv_freq is not None else 0, q_scale, k_scale, stream))
     register_op("memory_gates", entry_point="wllm_memory_gates",
-                argtypes=[c_void_p, c_longlong, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_longlong,
-                          c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
-                launch=lambda fn, stream, gates, i_bias, f_bias, qk, state, carried_offset, seg_q_start, seg_q_len,
-                state_slots, steps, heads, head_dim, cap, den_eps: fn(
-                    p(gates), gates.stride(0), p(i_bias), p(f_bias), float(cap) if cap else 0.0, den_eps, p(qk), p(state),
-                    state.stride(0), carried_offset, p(seg_q_start), p(seg_q_len), p(state_slots), p(steps), bf(gates),
-                    gates.shape[0], seg_q_start.shape[0], heads, head_dim, stream))
+                argtypes=[c_void_p, c_longlong, c_void_p, c_void_p, c_float, c_void_p, c_longlong, c_longlong, c_void_p,
+                          c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, gates, i_bias, f_bias, state, m_offset, seg_q_start, seg_q_len, state_slots, steps,
+                heads, cap: fn(
+                    p(gates), gates.stride(0), p(i_bias), p(f_bias), float(cap) if cap else 0.0, p(state), state.stride(0),
+                    m_offset, p(seg_q_start), p(seg_q_len), p(state_slots), p(steps), bf(gates), gates.shape[0],
+                    seg_q_start.shape[0], heads, stream))
     register_op("memory_scan", entry_point="wllm_memory_scan",
-                argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p,
-                          c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_longlong, c_longlong, c_void_p,
+                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
                 launch=lambda fn, stream, qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads,
-                head_dim, value_dim: fn(
-                    p(qk), p(v), v.stride(0), p(steps), p(decays), p(state), state.stride(0), p(seg_q_start), p(seg_q_len),
-                    p(state_slots), p(y), bf(v), v.shape[0], seg_q_start.shape[0], heads, head_dim, value_dim, stream))
+                head_dim, value_dim, nq=None, n_offset=0: fn(
+                    p(qk), p(v), v.stride(0), p(steps), p(decays), p(state), state.stride(0), n_offset, p(seg_q_start),
+                    p(seg_q_len), p(state_slots), p(y), p(nq), bf(v), v.shape[0], seg_q_start.shape[0], heads, head_dim,
+                    value_dim, stream))
     register_op("head_norm_gate", entry_point="wllm_head_norm_gate",
-                argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int,
-                          c_float, c_float, c_void_p],
-                launch=lambda fn, stream, y, gate, weight, out, heads, eps, activation, scale: fn(
-                    p(y), p(gate), gate.stride(0), p(weight), p(out), out.stride(0), bf(gate), GATE_KINDS[activation],
-                    y.shape[0], heads, y.shape[1] // heads, eps, scale, stream))
+                argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_float, c_int,
+                          c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
+                launch=lambda fn, stream, y, gate, weight, out, heads, eps, activation, scale, nq=None, floor=None,
+                den_eps=0.0: fn(
+                    p(y), p(gate), gate.stride(0), p(weight), p(out), out.stride(0), p(nq), p(floor), den_eps, bf(gate),
+                    GATE_KINDS[activation], y.shape[0], heads, y.shape[1] // heads, eps, scale, stream))
     register_op("moe_route", entry_point="wllm_moe_route",
                 argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                           c_void_p],
                 launch=lambda fn, stream, x, router, ids, weights, groups, keep, eps: fn(
                     p(x), p(router), p(ids), p(weights), bf(x), x.shape[0], x.shape[1], router.shape[0], ids.shape[1], groups,
                     keep, eps, stream))
-    register_op("moe_plan", entry_point="wllm_moe_plan", argtypes=[c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
-                launch=lambda fn, stream, ids, plan, experts: fn(
-                    p(ids), p(plan), ids.numel(), experts, moe_max_tiles(ids.numel(), experts), stream))
+    register_op("moe_plan", entry_point="wllm_moe_plan", argtypes=[c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, ids, plan, experts, tile_rows=MOE_TILE_ROWS: fn(
+                    p(ids), p(plan), ids.numel(), experts, moe_max_tiles(ids.numel(), experts, tile_rows), tile_rows, stream))
     register_op("moe_experts_up", entry_point="wllm_moe_up",
                 argtypes=[c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
                 launch=lambda fn, stream, x, w, plan, act, top, activation: fn(
@@ -1251,6 +1284,15 @@ def _register_own() -> None:
                 launch=lambda fn, stream, act, w, plan, weights, out: fn(
                     p(act), p(w), p(plan), moe_max_tiles(act.shape[0], w.shape[0]), p(weights), p(out), bf(act),
                     weights.shape[0], act.shape[1], w.shape[1], weights.shape[1], stream))
-
+    tiles = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+             c_void_p]
+    register_op("moe_experts_up_tiled", entry_point="wllm_moe_tiles", argtypes=tiles,
+                launch=lambda fn, stream, x, w, plan, act, top, activation: fn(
+                    p(x), p(w), p(plan), moe_max_tiles(act.shape[0], w.shape[0], MOE_BIG_TILE_ROWS), p(act), p(None), p(None),
+                    ACTIVATIONS[activation], x.shape[0], act.shape[1], x.shape[1], top, x.shape[0], stream))
+    register_op("moe_experts_down_tiled", entry_point="wllm_moe_tiles", argtypes=tiles,
+                launch=lambda fn, stream, act, w, plan, weights, out: fn(
+                    p(act), p(w), p(plan), moe_max_tiles(act.shape[0], w.shape[0], MOE_BIG_TILE_ROWS), p(None), p(out),
+                    p(weights), -1, act.shape[0], w.shape[1], act.shape[1], weights.shape[1], weights.shape[0], stream))
 
 _register_own()

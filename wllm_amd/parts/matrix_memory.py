@@ -9,7 +9,9 @@
 With `gating` "decay", a_t is the head's fixed decay and b_t = den_t = 1 (retention).  With "exponential",
 the two gate projections give a log input gate and a log forget gate (both bent under a cap), a running
 maximum m holds the exponentials in range, a normaliser n_t = a_t n_(t-1) + b_t k_t is carried beside S and
-den_t = max(|n_t . q_t|, exp(-m_t)) + den_eps (the matrix memory of an mLSTM).
+den_t = max(|n_t . q_t|, exp(-m_t)) + den_eps (the matrix memory of an mLSTM).  The normaliser is one more
+column of the memory (a value that is always 1), so the recurrence's kernel carries it and leaves n . q beside
+the columns' sums; the kernel that norms the heads divides by den first.
 
 A request carries S (and n, m) from step to step in one float32 state row of the cache manager
 ([heads * head_dim * value_dim], then [heads * head_dim], then [heads]; zeroed at admission: all three
@@ -125,17 +127,21 @@ class MatrixMemoryMixer:
         qk = ctx.buffer("memory_qk", (2, n, self.qk_width), torch.float32)
         ops.memory_inputs(row, ctx.positions, self.position.inv_freq, qk, heads=s.num_heads, head_dim=s.head_dim,
                           q_scale=s.q_scale, k_scale=s.k_scale)
-        steps = None
+        steps = nq = None
         if self.exponential:
+            # the normaliser lies behind the memory in the request's row, the running maxima behind it
+            n_offset = self.memory_size
             steps = ctx.buffer("memory_steps", (3, n, s.num_heads), torch.float32)
-            ops.memory_gates(row[:, self.gates_offset:self.gates_offset + 2 * s.num_heads], self.i_bias, self.f_bias, qk,
-                             state, self.memory_size, ctx.seg_q_start, ctx.seg_q_len, ctx.state_slots, steps,
-                             heads=s.num_heads, head_dim=s.head_dim, cap=s.gate_cap, den_eps=s.den_eps)
+            nq = ctx.buffer("memory_nq", (n, s.num_heads), torch.float32)
+            ops.memory_gates(row[:, self.gates_offset:self.gates_offset + 2 * s.num_heads], self.i_bias, self.f_bias, state,
+                             n_offset + self.qk_width, ctx.seg_q_start, ctx.seg_q_len, ctx.state_slots, steps,
+                             heads=s.num_heads, cap=s.gate_cap)
         y = ctx.buffer("memory_y", (n, self.v_width), torch.float32)
         ops.memory_scan(qk, row[:, self.v_offset:self.v_offset + self.v_width], steps, self.decays, state,
                         ctx.seg_q_start, ctx.seg_q_len, ctx.state_slots, y, heads=s.num_heads, head_dim=s.head_dim,
-                        value_dim=s.value_dim)
+                        value_dim=s.value_dim, nq=nq, n_offset=self.memory_size if self.exponential else 0)
         out = product_input if product_input is not None else ctx.buffer("memory_out", (n, self.v_width), h.dtype)
         ops.head_norm_gate(y, row[:, self.g_offset:self.g_offset + self.v_width], self.norm_w, out, heads=s.num_heads,
-                           eps=s.norm_eps, activation=s.gate_activation, scale=s.output_scale)
+                           eps=s.norm_eps, activation=s.gate_activation, scale=s.output_scale, nq=nq,
+                           floor=steps[2] if self.exponential else None, den_eps=s.den_eps if self.exponential else 0.0)
         return Product("mixer_out", out, self.w_o, self.t_o)

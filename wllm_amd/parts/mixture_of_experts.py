@@ -7,8 +7,10 @@
 
 The experts' matrices are stacked at load ([experts, 2 * ff, width]: an expert's gate rows, then its up
 rows; [experts, width, ff]).  A step routes its tokens, sorts the (token, expert) pairs by expert on the
-device (`ops.moe_plan`: tiles of 16 rows of one expert) and runs the two products expert by expert on
-the matrix cores, each tile with its expert's weights.  The second product weighs a pair's result and
+device (`ops.moe_plan`: tiles of rows of one expert) and runs the two products expert by expert on
+the matrix cores, each tile with its expert's weights: tiles of 16 rows past which an expert's weights
+stream where the experts get few rows each (decoded tokens), tiles of 128 rows through shared memory
+where they get many (a prompt's portion).  The second product weighs a pair's result and
 leaves it in the slice of its slot of a float32 stack [top, tokens, width], which whoever adds the
 feed-forward to the stream (the next norm kernel) adds in order: the weighted sum is formed in float32
 and takes no pass of its own.  Nothing of the routing is read on the host.
@@ -85,10 +87,11 @@ class MixtureOfExperts:
         ids = ctx.buffer("moe_ids", (n, s.top), torch.int32)
         weights = ctx.buffer("moe_weights", (n, s.top), torch.float32)
         ops.moe_route(h, self.w_router, ids, weights, groups=s.num_groups, keep=s.keep_groups, eps=s.weight_eps)
-        plan = ctx.buffer("moe_plan", (ops.moe_plan_size(n * s.top, s.num_experts),), torch.int32)
-        ops.moe_plan(ids, plan, s.num_experts)
+        rows = ops.moe_tile_rows(n * s.top, s.num_experts, h.dtype, s.hidden_size, s.intermediate_size)
+        plan = ctx.buffer("moe_plan", (ops.moe_plan_size(n * s.top, s.num_experts, rows),), torch.int32)
+        ops.moe_plan(ids, plan, s.num_experts, rows)
         act = ctx.buffer("moe_act", (n * s.top, s.intermediate_size), h.dtype)
-        ops.moe_experts_up(h, self.w_up, plan, act, s.top, s.activation)
+        ops.moe_experts_up(h, self.w_up, plan, act, s.top, s.activation, rows)
         out = ctx.buffer("moe_out", (s.top, n, s.hidden_size), torch.float32)
-        ops.moe_experts_down(act, self.w_down, plan, weights, out)
+        ops.moe_experts_down(act, self.w_down, plan, weights, out, rows)
         return out
