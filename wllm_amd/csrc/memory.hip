@@ -138,38 +138,40 @@ WLLM_API int wllm_memory_gates(const void* gates, long long gates_stride, const 
 // ---- the recurrence itself.  A workgroup owns (head, segment, 16 columns of P) and walks the segment's
 // tokens in order.  D is cut into 32 slices: a lane is (column, one of four slices), a wavefront four
 // slices, the workgroup's eight wavefronts all of them; a lane keeps its R rows of its column of S in
-// registers.  Tokens are staged 16 at a time through shared memory (q, k, v, a, b); a token's sum is
-// the slices' partial sums added in a fixed order (within the wavefront, then wavefront by wavefront),
-// so it has the same bits whether the token came alone or inside a prompt.  With `steps` the column behind
-// the last (p = P) is the normaliser: its value is 1 for every token, its rows lie at `n_offset` of the
-// request's row, and its sums go to `nq` [tokens, heads]. ----
+// registers.  Tokens go 16 at a time through shared memory (q, k, v, a, b), the next 16 fetched into registers
+// while these are walked; a token's sum is the slices' partial sums added in a fixed order (within the
+// wavefront, then wavefront by wavefront), so it has the same bits whether the token came alone or inside a
+// prompt.  With `steps` the column behind the last (p = P) is the normaliser: its value is 1 for every token,
+// its rows lie at `n_offset` of the request's row, and its sums go to `nq` [tokens, heads]. ----
 constexpr int kMemTokens = 16;
 constexpr int kMemWaves = 8;
 constexpr int kMemCols = 16;
 constexpr int kMemSlices = kMemWaves * (kWave / kMemCols);
+constexpr int kMemThreads = kWave * kMemWaves;
 
 template <typename T, int R>
-__global__ void __launch_bounds__(kWave * kMemWaves)
+__global__ void __launch_bounds__(kMemThreads)
 memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long long v_stride, const float* __restrict__ steps,
                    const float* __restrict__ decays, float* __restrict__ state, long long state_stride, long long n_offset,
                    const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len, const int* __restrict__ state_slots,
                    float* __restrict__ y, float* __restrict__ nq, int tokens, int heads, int d, int p_dim) {
-    extern __shared__ __align__(16) float smem[];
+    constexpr int kRow = kMemSlices * R;                   // a token's row of q (and of k) in shared memory: d and zeros
+    constexpr int kPasses = kMemTokens * kRow / kMemThreads;      // elements of q (and of k) a thread stages: R
+    constexpr int kRowsPass = kMemThreads / kRow;          // tokens a pass covers
+    __shared__ __align__(16) float q_s[kMemTokens * kRow];
+    __shared__ __align__(16) float k_s[kMemTokens * kRow];
+    __shared__ float v_s[kMemTokens * kMemCols];
+    __shared__ float a_s[kMemTokens], b_s[kMemTokens];
+    __shared__ float part_s[kMemTokens * kMemWaves * kMemCols];
     const int h = blockIdx.x, seg = blockIdx.y, p0 = blockIdx.z * kMemCols;
     const int q_len = seg_q_len[seg], q_start = seg_q_start[seg];
     if (q_len <= 0) return;
-    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int tid = threadIdx.x;
+    const int lane = tid % kWave, wave = tid / kWave;
     const int col = lane % kMemCols, slice = wave * (kWave / kMemCols) + lane / kMemCols;
     const int p = p0 + col;
     const bool norm_col = steps != nullptr && p == p_dim;
     const bool live = p < p_dim || norm_col;
-    const int d_pad = (d + 3) / 4 * 4;
-    float* q_s = smem;                                   // [kMemTokens][d_pad]
-    float* k_s = q_s + kMemTokens * d_pad;               // [kMemTokens][d_pad]
-    float* v_s = k_s + kMemTokens * d_pad;               // [kMemTokens][kMemCols]
-    float* a_s = v_s + kMemTokens * kMemCols;            // [kMemTokens]
-    float* b_s = a_s + kMemTokens;
-    float* part_s = b_s + kMemTokens;                    // [kMemTokens][kMemWaves][kMemCols]
     const size_t width = static_cast<size_t>(heads) * d, all = static_cast<size_t>(tokens) * heads;
     float* request = state + static_cast<size_t>(state_slots[seg]) * state_stride;
     // this lane's column of the state: rows p_dim apart in S, or the normaliser's rows one after the other
@@ -180,44 +182,79 @@ memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long l
 #pragma unroll
     for (int i = 0; i < R; ++i) s[i] = (live && n0 + i < d) ? s_rows[static_cast<size_t>(n0 + i) * s_step] : 0.f;
     const float fixed = decays ? decays[h] : 1.f;
+
+    // what this thread stages of every 16 tokens: element `sj` of the rows of tokens st, st + kRowsPass, ... of q and of
+    // k (zeros beyond d: a row of S that is not there stays zero and adds nothing), one value of v, one token's a and b
+    const int sj = tid % kRow, st = tid / kRow;
+    const int vt = tid / kMemCols, vc = tid % kMemCols;
+    float q_r[kPasses], k_r[kPasses], v_r = 0.f, a_r = 1.f, b_r = 1.f;
+    auto fetch = [&](int t0) {
+        const int count = min(kMemTokens, q_len - t0);
+#pragma unroll
+        for (int u = 0; u < kPasses; ++u) {
+            const int t = st + u * kRowsPass;
+            q_r[u] = k_r[u] = 0.f;
+            if (sj < d && t < count) {
+                const size_t at = static_cast<size_t>(q_start + t0 + t) * width + static_cast<size_t>(h) * d + sj;
+                q_r[u] = qk[at];
+                k_r[u] = qk[static_cast<size_t>(tokens) * width + at];
+            }
+        }
+        if (tid < kMemTokens * kMemCols) {
+            v_r = 0.f;
+            if (vt < count) {
+                if (p0 + vc < p_dim)
+                    v_r = to_float(v[static_cast<size_t>(q_start + t0 + vt) * v_stride + static_cast<size_t>(h) * p_dim + p0 + vc]);
+                else if (steps != nullptr && p0 + vc == p_dim)
+                    v_r = 1.f;
+            }
+        }
+        if (tid < count) {
+            const size_t at = static_cast<size_t>(q_start + t0 + tid) * heads + h;
+            a_r = steps ? steps[at] : fixed;
+            b_r = steps ? steps[all + at] : 1.f;
+        }
+    };
+    auto place = [&]() {
+#pragma unroll
+        for (int u = 0; u < kPasses; ++u) {
+            q_s[(st + u * kRowsPass) * kRow + sj] = q_r[u];
+            k_s[(st + u * kRowsPass) * kRow + sj] = k_r[u];
+        }
+        if (tid < kMemTokens * kMemCols) v_s[tid] = v_r;
+        if (tid < kMemTokens) {
+            a_s[tid] = a_r;
+            b_s[tid] = b_r;
+        }
+    };
+    auto token = [&](int t) {
+        const float a = a_s[t], bv = b_s[t] * v_s[t * kMemCols + col];
+        const float* kt = k_s + t * kRow + n0;
+        const float* qt = q_s + t * kRow + n0;
+        float part = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            s[i] = fmaf(a, s[i], bv * kt[i]);
+            part = fmaf(s[i], qt[i], part);
+        }
+        part = sum_across(sum_across(part, 32), 16);      // the wavefront's four slices of this column
+        if (lane < kMemCols) part_s[(t * kMemWaves + wave) * kMemCols + col] = part;
+    };
+
+    fetch(0);
     for (int t0 = 0; t0 < q_len; t0 += kMemTokens) {
         const int count = min(kMemTokens, q_len - t0);
-        __syncthreads();                                 // the chunk before is read out
-        for (int e = threadIdx.x; e < count * d; e += blockDim.x) {
-            const int t = e / d, j = e - t * d;
-            const size_t at = static_cast<size_t>(q_start + t0 + t) * width + static_cast<size_t>(h) * d + j;
-            q_s[t * d_pad + j] = qk[at];
-            k_s[t * d_pad + j] = qk[static_cast<size_t>(tokens) * width + at];
-        }
-        for (int e = threadIdx.x; e < count * kMemCols; e += blockDim.x) {
-            const int t = e / kMemCols, c = e % kMemCols;
-            v_s[e] = p0 + c < p_dim
-                         ? to_float(v[static_cast<size_t>(q_start + t0 + t) * v_stride + static_cast<size_t>(h) * p_dim + p0 + c])
-                         : (steps != nullptr && p0 + c == p_dim ? 1.f : 0.f);
-        }
-        if (threadIdx.x < count) {
-            const size_t at = static_cast<size_t>(q_start + t0 + threadIdx.x) * heads + h;
-            a_s[threadIdx.x] = steps ? steps[at] : fixed;
-            b_s[threadIdx.x] = steps ? steps[all + at] : 1.f;
-        }
+        place();
         __syncthreads();
-        for (int t = 0; t < count; ++t) {
-            const float a = a_s[t], bv = b_s[t] * v_s[t * kMemCols + col];
-            const float* kt = k_s + t * d_pad + n0;
-            const float* qt = q_s + t * d_pad + n0;
-            float part = 0.f;
+        if (t0 + kMemTokens < q_len) fetch(t0 + kMemTokens);     // on their way while these 16 are walked
+        if (count == kMemTokens) {
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                if (n0 + i < d) {
-                    s[i] = fmaf(a, s[i], bv * kt[i]);
-                    part = fmaf(s[i], qt[i], part);
-                }
-            }
-            part = sum_across(sum_across(part, 32), 16);      // the wavefront's four slices of this column
-            if (lane < kMemCols) part_s[(t * kMemWaves + wave) * kMemCols + col] = part;
+            for (int t = 0; t < kMemTokens; ++t) token(t);
+        } else {
+            for (int t = 0; t < count; ++t) token(t);
         }
         __syncthreads();
-        for (int e = threadIdx.x; e < count * kMemCols; e += blockDim.x) {
+        for (int e = tid; e < count * kMemCols; e += kMemThreads) {
             const int t = e / kMemCols, l = e % kMemCols;
             if (p0 + l > p_dim || (p0 + l == p_dim && steps == nullptr)) continue;
             float total = part_s[(t * kMemWaves) * kMemCols + l];
@@ -226,6 +263,8 @@ memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long l
             if (p0 + l == p_dim) nq[static_cast<size_t>(q_start + t0 + t) * heads + h] = total;
             else y[static_cast<size_t>(q_start + t0 + t) * heads * p_dim + static_cast<size_t>(h) * p_dim + p0 + l] = total;
         }
+        // (the next round's `place` writes q, k, v, a, b, which nobody reads any more; its barrier stands between
+        // these reads of the partial sums and the next writes to them)
     }
     if (live) {
 #pragma unroll
@@ -245,16 +284,12 @@ WLLM_API int wllm_memory_scan(const float* qk, const void* v, long long v_stride
     if (heads <= 0 || d <= 0 || d > 8 * kMemSlices || p_dim <= 0) return -1;
     if (segments > 65535 || (p_dim + kMemCols) / kMemCols > 65535) return -1;
     const int r = (d + kMemSlices - 1) / kMemSlices;
-    const int d_pad = (d + 3) / 4 * 4;
     const int columns = p_dim + (steps ? 1 : 0);
     const dim3 grid(heads, segments, (columns + kMemCols - 1) / kMemCols);
-    const size_t smem = sizeof(float) * (2 * kMemTokens * d_pad + kMemTokens * kMemCols + 2 * kMemTokens +
-                                         kMemTokens * kMemWaves * kMemCols);
-#define LAUNCH(T, R)                                                                                                  \
-    memory_scan_kernel<T, R><<<grid, kWave * kMemWaves, smem, stream>>>(qk, static_cast<const T*>(v), v_stride, steps, \
-                                                                        decays, state, state_stride, n_offset,       \
-                                                                        seg_q_start, seg_q_len, state_slots, y, nq,  \
-                                                                        tokens, heads, d, p_dim)
+#define LAUNCH(T, R)                                                                                                \
+    memory_scan_kernel<T, R><<<grid, kMemThreads, 0, stream>>>(qk, static_cast<const T*>(v), v_stride, steps, decays, \
+                                                               state, state_stride, n_offset, seg_q_start, seg_q_len, \
+                                                               state_slots, y, nq, tokens, heads, d, p_dim)
 #define LAUNCH_R(T)                        \
     if (r <= 1) LAUNCH(T, 1);              \
     else if (r <= 2) LAUNCH(T, 2);         \
