@@ -455,7 +455,7 @@ class EmulatedKernels:
             at = 1 + max_tiles + 16 * t
             yield int(plan[1 + t]), [a for a in plan[at:at + 16].tolist() if a >= 0]
 
-    def moe_experts_up(self, x, w, plan, act, top, activation):
+    def moe_experts_up(self, x, w, plan, act, top, activation, tiles=None):
         self._count("moe_experts_up")
         ff = w.shape[1] // 2
         for e, rows in self._plan_rows(plan, w.shape[0], act.shape[0]):
@@ -467,7 +467,7 @@ class EmulatedKernels:
                 z = z * torch.sigmoid(z)
             act[rows] = (z * u).to(act.dtype)
 
-    def moe_experts_down(self, act, w, plan, weights, out):
+    def moe_experts_down(self, act, w, plan, weights, out, tiles=None):
         self._count("moe_experts_down")
         n, top = weights.shape
         flat = weights.reshape(-1)

@@ -219,7 +219,7 @@ def test_segments_of_a_batch_keep_their_own_memories(dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n,width,ff,count,top,groups,keep", [
-    (1, 64, 48, 6, 2, 3, 2), (7, 48, 24, 5, 3, 5, 5), (40, 96, 70, 8, 3, 4, 2), (300, 128, 96, 16, 4, 4, 2), (33, 36, 10, 1, 1, 1, 1),
+    (1, 64, 48, 6, 2, 3, 2), (9, 128, 256, 5, 2, 1, 1), (7, 48, 24, 5, 3, 5, 5), (40, 96, 70, 8, 3, 4, 2), (300, 128, 96, 16, 4, 4, 2), (33, 36, 10, 1, 1, 1, 1),
     (90, 64, 32, 12, 1, 3, 1), (5, 256, 130, 4, 4, 2, 2), (130, 50, 16, 9, 6, 3, 2),
     (300, 128, 192, 4, 2, 2, 1), (700, 64, 64, 3, 1, 1, 1), (450, 192, 128, 6, 3, 3, 2)])     # bfloat16: tiles of 128 rows
 def test_the_router_and_the_experts(dtype, n, width, ff, count, top, groups, keep):
@@ -263,9 +263,14 @@ def test_the_router_and_the_experts(dtype, n, width, ff, count, top, groups, kee
         assert all(int(flat_ids[a]) == e for a in rows[tile * t:tile * t + tile].tolist() if a >= 0)
     stack = lambda names: torch.stack([torch.cat([w[f"f.e{e}.{x}"] for x in names]) for e in range(count)]).to(dtype).to(DEV)
     act = torch.zeros(n * top, ff, dtype=dtype, device=DEV)
-    ops.moe_experts_up(x, stack(("gate", "up")), plan, act, top, "silu", tile)
+    w_up, w_down = stack(("gate", "up")), stack(("down",))
+    # the weights' tile-major copies, where the few-row kernels take them
+    streamed = dtype == torch.bfloat16 and width % 32 == 0 and ff % 32 == 0
+    t_up = ops.tile_weight(w_up.view(-1, width)) if streamed else None
+    t_down = ops.tile_weight(w_down.view(-1, ff)) if streamed else None
+    ops.moe_experts_up(x, w_up, plan, act, top, "silu", tile, t_up)
     out = torch.full((top, n, width), float("nan"), dtype=torch.float32, device=DEV)
-    ops.moe_experts_down(act, stack(("down",)), plan, wts, out, tile)
+    ops.moe_experts_down(act, w_down, plan, wts, out, tile, t_down)
     rounding = plain.to_bfloat16 if dtype == torch.bfloat16 else plain.same
     want = plain.mixture_of_experts(h.double(), w, "f.", c, rounding)
     got = out.sum(0)

@@ -99,13 +99,19 @@ memory_gates_kernel(const T* __restrict__ gates, long long gates_stride, const f
             lf = log_sigmoid(bent(to_float(g[heads + h]) + bf, cap));
         }
         float m_before = 0.f, m_mine = 0.f;
-        for (int t = 0; t < count; ++t) {
+        auto follow = [&](int t) {
             const float m_new = fmaxf(from_lane(lf, t) + m, from_lane(li, t));
             if (lane == t) {
                 m_before = m;
                 m_mine = m_new;
             }
             m = m_new;
+        };
+        if (count == kWave) {
+#pragma unroll
+            for (int t = 0; t < kWave; ++t) follow(t);
+        } else {
+            for (int t = 0; t < count; ++t) follow(t);
         }
         if (lane < count) {
             const size_t at = static_cast<size_t>(q_start + t0 + lane) * heads + h;

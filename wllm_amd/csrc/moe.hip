@@ -258,10 +258,13 @@ template <> struct MoeFrag<float> {
 
 // act[a, c] = activation(x[token(a)] . Wg[e][c]) * (x[token(a)] . Wu[e][c]); w [experts, 2 * ff, K]: an
 // expert's gate rows, then its up rows.  Grid (tiles, bands of 64 columns); a wavefront 16 columns.
+// `tiles`: the weights' tile-major copy (bfloat16: per band of 16 rows of the stacked [experts * 2 * ff, K] matrix and
+// step of 32 keys one KiB in lane order, as `wllm_tile_weight` writes it; ff a multiple of 16), or null: then a
+// wavefront's load of a fragment is one contiguous KiB instead of 16 pieces a row apart.
 template <typename T, int ACT>
 __global__ void __launch_bounds__(256)
-moe_up_kernel(const T* __restrict__ x, const T* __restrict__ w, const int* __restrict__ plan, int max_tiles,
-              T* __restrict__ act, int K, int ff, int top) {
+moe_up_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ tiles, const int* __restrict__ plan,
+              int max_tiles, T* __restrict__ act, int K, int ff, int top) {
     const int tile = blockIdx.x;
     if (tile >= plan[0]) return;
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -277,7 +280,25 @@ moe_up_kernel(const T* __restrict__ x, const T* __restrict__ w, const int* __res
     const T* wu = wg + static_cast<size_t>(ff) * K;
     float4_t acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
     constexpr int kChunk = MoeFrag<T>::kChunk, kPer = MoeFrag<T>::kPer;
-    if (K % (4 * kChunk) == 0) {
+    if (tiles != nullptr && K % (4 * kChunk) == 0) {
+        const size_t per_band = static_cast<size_t>(K / kChunk) * kWave * kPer;        // elements of a band's tiles
+        const T* tg = tiles + (static_cast<size_t>(e) * 2 * ff + c0) / 16 * per_band + lane * kPer;
+        const T* tu = tiles + (static_cast<size_t>(e) * 2 * ff + ff + c0) / 16 * per_band + lane * kPer;
+        for (int k0 = 0; k0 < K; k0 += 4 * kChunk) {
+            MoeFrag<T> fx[4], fg[4], fu[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                fx[u].whole(xr + k0 + u * kChunk + g * kPer);
+                fg[u].template whole<true>(tg + static_cast<size_t>(k0 / kChunk + u) * kWave * kPer);
+                fu[u].template whole<true>(tu + static_cast<size_t>(k0 / kChunk + u) * kWave * kPer);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                acc_g = MoeFrag<T>::mma(fg[u], fx[u], acc_g);
+                acc_u = MoeFrag<T>::mma(fu[u], fx[u], acc_u);
+            }
+        }
+    } else if (K % (4 * kChunk) == 0) {
         // every fragment is whole (rows that stand for nothing read row 0, and their sums are dropped); four
         // chunks' loads are asked for before the first product
         for (int k0 = g * kPer; k0 < K; k0 += 4 * kChunk) {
@@ -314,15 +335,16 @@ moe_up_kernel(const T* __restrict__ x, const T* __restrict__ w, const int* __res
     }
 }
 
-WLLM_API int wllm_moe_up(const void* x, const void* w, const int* plan, int max_tiles, void* act, int is_bf16, int activation,
-                         int K, int ff, int top, hipStream_t stream) {
+WLLM_API int wllm_moe_up(const void* x, const void* w, const void* tiles, const int* plan, int max_tiles, void* act, int is_bf16,
+                         int activation, int K, int ff, int top, hipStream_t stream) {
     if (max_tiles <= 0) return 0;
     if (K <= 0 || ff <= 0 || top <= 0 || activation < 0 || activation >= kActivations || (ff + 63) / 64 > 65535) return -1;
+    if (tiles && (!is_bf16 || ff % 16 || K % 32)) return -1;
     const dim3 grid(max_tiles, (ff + 63) / 64);
 #define LAUNCH(T)                                                                                                     \
     WLLM_BY_ACTIVATION(activation, (moe_up_kernel<T, ACT><<<grid, 256, 0, stream>>>(                                  \
-                                       static_cast<const T*>(x), static_cast<const T*>(w), plan, max_tiles,           \
-                                       static_cast<T*>(act), K, ff, top)))
+                                       static_cast<const T*>(x), static_cast<const T*>(w), static_cast<const T*>(tiles), \
+                                       plan, max_tiles, static_cast<T*>(act), K, ff, top)))
     if (is_bf16) { LAUNCH(bf16); } else { LAUNCH(float); }
 #undef LAUNCH
     return launch_status();
@@ -331,8 +353,9 @@ WLLM_API int wllm_moe_up(const void* x, const void* w, const int* plan, int max_
 // out[a % top][a / top][c] = weight[a] * (act[a] . Wd[e][c]); w [experts, width, ff]; out float32 [top, tokens, width].
 template <typename T>
 __global__ void __launch_bounds__(256)
-moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w, const int* __restrict__ plan, int max_tiles,
-                const float* __restrict__ weights, float* __restrict__ out, int tokens, int ff, int width, int top) {
+moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w, const T* __restrict__ tiles, const int* __restrict__ plan,
+                int max_tiles, const float* __restrict__ weights, float* __restrict__ out, int tokens, int ff, int width,
+                int top) {
     const int tile = blockIdx.x;
     if (tile >= plan[0]) return;
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -347,7 +370,20 @@ moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w, const int* _
     const T* wd = w + (static_cast<size_t>(e) * width + (w_live ? c0 + i : 0)) * ff;
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
     constexpr int kChunk = MoeFrag<T>::kChunk, kPer = MoeFrag<T>::kPer;
-    if (ff % (4 * kChunk) == 0) {
+    if (tiles != nullptr && ff % (4 * kChunk) == 0) {
+        const size_t per_band = static_cast<size_t>(ff / kChunk) * kWave * kPer;
+        const T* td = tiles + (static_cast<size_t>(e) * width + c0) / 16 * per_band + lane * kPer;
+        for (int k0 = 0; k0 < ff; k0 += 4 * kChunk) {
+            MoeFrag<T> fx[4], fw[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                fx[u].whole(xr + k0 + u * kChunk + g * kPer);
+                fw[u].template whole<true>(td + static_cast<size_t>(k0 / kChunk + u) * kWave * kPer);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc = MoeFrag<T>::mma(fw[u], fx[u], acc);
+        }
+    } else if (ff % (4 * kChunk) == 0) {
         for (int k0 = g * kPer; k0 < ff; k0 += 4 * kChunk) {
             MoeFrag<T> fx[4], fw[4];
 #pragma unroll
@@ -377,17 +413,20 @@ moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w, const int* _
     }
 }
 
-WLLM_API int wllm_moe_down(const void* act, const void* w, const int* plan, int max_tiles, const float* weights, float* out,
-                           int is_bf16, int tokens, int ff, int width, int top, hipStream_t stream) {
+WLLM_API int wllm_moe_down(const void* act, const void* w, const void* tiles, const int* plan, int max_tiles,
+                           const float* weights, float* out, int is_bf16, int tokens, int ff, int width, int top,
+                           hipStream_t stream) {
     if (max_tiles <= 0 || tokens <= 0) return 0;
     if (ff <= 0 || width <= 0 || top <= 0 || (width + 63) / 64 > 65535) return -1;
+    if (tiles && (!is_bf16 || width % 16 || ff % 32)) return -1;
     const dim3 grid(max_tiles, (width + 63) / 64);
     if (is_bf16)
-        moe_down_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(act), static_cast<const bf16*>(w), plan,
-                                                        max_tiles, weights, out, tokens, ff, width, top);
+        moe_down_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(act), static_cast<const bf16*>(w),
+                                                        static_cast<const bf16*>(tiles), plan, max_tiles, weights, out, tokens,
+                                                        ff, width, top);
     else
-        moe_down_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(act), static_cast<const float*>(w), plan,
-                                                         max_tiles, weights, out, tokens, ff, width, top);
+        moe_down_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(act), static_cast<const float*>(w), nullptr,
+                                                         plan, max_tiles, weights, out, tokens, ff, width, top);
     return launch_status();
 }
 

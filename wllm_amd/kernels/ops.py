@@ -1073,11 +1073,19 @@ def _big_tiles(tile_rows: int, dtype, inner: int) -> bool:
     return False
 
 
+def _expert_tiles(tiles: Optional[torch.Tensor], w: torch.Tensor) -> None:
+    if tiles is not None:
+        _need(w.dtype == torch.bfloat16 and w.shape[1] % 16 == 0 and w.shape[2] % 32 == 0,
+              "tiles: bfloat16 experts of a multiple of 16 rows and of 32 keys")
+        _dense(tiles, "tiles", w.dtype, (w.numel(),))
+
+
 def moe_experts_up(x: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, act: torch.Tensor, top: int,
-                   activation: str, tile_rows: int = MOE_TILE_ROWS) -> None:
+                   activation: str, tile_rows: int = MOE_TILE_ROWS, tiles: Optional[torch.Tensor] = None) -> None:
     """act[a] = activation(x[a // top] Wg_e^T) * (x[a // top] Wu_e^T) for every assignment a of the plan (of tiles of
     `tile_rows` rows), e its expert.  x T [n, width]; w T [experts, 2 * ff, width]: an expert's gate rows, then its
-    up rows; act T [n * top, ff]; float32 sums."""
+    up rows; act T [n * top, ff]; float32 sums.  `tiles`: `tile_weight` of w as one matrix [experts * 2 * ff, width]
+    (ff a multiple of 16), which the kernel for tiles of 16 rows streams instead of w."""
     _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {sorted(ACTIVATIONS)}")
     _dense(x, "x", _ACT)
     _need(x.dim() == 2, "x: expected [n, width]")
@@ -1087,15 +1095,17 @@ def moe_experts_up(x: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, act: to
     experts, ff = w.shape[0], w.shape[1] // 2
     _dense(act, "act", x.dtype, (n * top, ff))
     _dense(plan, "plan", torch.int32, (moe_plan_size(n * top, experts, tile_rows),))
+    _need(tiles is None or ff % 16 == 0, "tiles: ff must be a multiple of 16")
+    _expert_tiles(tiles, w)
     if n:
         if _big_tiles(tile_rows, x.dtype, width):
             call("moe_experts_up_tiled", x, w, plan, act, int(top), activation)
         else:
-            call("moe_experts_up", x, w, plan, act, int(top), activation)
+            call("moe_experts_up", x, w, plan, act, int(top), activation, tiles)
 
 
 def moe_experts_down(act: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, weights: torch.Tensor,
-                     out: torch.Tensor, tile_rows: int = MOE_TILE_ROWS) -> None:
+                     out: torch.Tensor, tile_rows: int = MOE_TILE_ROWS, tiles: Optional[torch.Tensor] = None) -> None:
     """out[a % top][a // top] = weights.flat[a] * (act[a] Wd_e^T) for every assignment a of the plan: the
     experts' weighted results as a stack of `top` float32 partial sums over the tokens.  act T [n * top, ff];
     w T [experts, width, ff]; weights float32 [n, top]; out float32 [top, n, width]."""
@@ -1108,11 +1118,12 @@ def moe_experts_down(act: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, wei
     _need(w.dim() == 3 and w.shape[2] == act.shape[1], "w: expected [experts, width, ff]")
     _dense(out, "out", torch.float32, (top, n, w.shape[1]))
     _dense(plan, "plan", torch.int32, (moe_plan_size(n * top, w.shape[0], tile_rows),))
+    _expert_tiles(tiles, w)
     if n:
         if _big_tiles(tile_rows, act.dtype, act.shape[1]):
             call("moe_experts_down_tiled", act, w, plan, weights, out)
         else:
-            call("moe_experts_down", act, w, plan, weights, out)
+            call("moe_experts_down", act, w, plan, weights, out, tiles)
 
 
 # ---- the framework's own operations that go through the same door as a part's ------------------
@@ -1274,15 +1285,15 @@ def _register_own() -> None:
                 launch=lambda fn, stream, ids, plan, experts, tile_rows=MOE_TILE_ROWS: fn(
                     p(ids), p(plan), ids.numel(), experts, moe_max_tiles(ids.numel(), experts, tile_rows), tile_rows, stream))
     register_op("moe_experts_up", entry_point="wllm_moe_up",
-                argtypes=[c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
-                launch=lambda fn, stream, x, w, plan, act, top, activation: fn(
-                    p(x), p(w), p(plan), moe_max_tiles(act.shape[0], w.shape[0]), p(act), bf(x), ACTIVATIONS[activation],
-                    x.shape[1], act.shape[1], top, stream))
+                argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, x, w, plan, act, top, activation, tiles=None: fn(
+                    p(x), p(w), p(tiles), p(plan), moe_max_tiles(act.shape[0], w.shape[0]), p(act), bf(x),
+                    ACTIVATIONS[activation], x.shape[1], act.shape[1], top, stream))
     register_op("moe_experts_down", entry_point="wllm_moe_down",
-                argtypes=[c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                           c_void_p],
-                launch=lambda fn, stream, act, w, plan, weights, out: fn(
-                    p(act), p(w), p(plan), moe_max_tiles(act.shape[0], w.shape[0]), p(weights), p(out), bf(act),
+                launch=lambda fn, stream, act, w, plan, weights, out, tiles=None: fn(
+                    p(act), p(w), p(tiles), p(plan), moe_max_tiles(act.shape[0], w.shape[0]), p(weights), p(out), bf(act),
                     weights.shape[0], act.shape[1], w.shape[1], weights.shape[1], stream))
     tiles = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
              c_void_p]

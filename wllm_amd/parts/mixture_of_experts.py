@@ -41,6 +41,7 @@ class MixtureOfExperts:
             raise ValueError(f"top ({spec.top}): at most the experts of the kept groups")
         self.spec = spec
         self.w_router = self.w_up = self.w_down = None
+        self.t_up = self.t_down = None          # the stacks' tile-major copies, which the few-row kernels stream
 
     def _names(self, e: int) -> tuple:
         s = self.spec
@@ -68,6 +69,11 @@ class MixtureOfExperts:
         self.w_up = fetch.to_device(torch.stack(ups).contiguous())
         self.w_down = fetch.to_device(torch.stack(downs).contiguous())
         self.w_router = fetch.to_device(fetch.vector(s.router_weight))
+        if (getattr(fetch, "tiled_copies", False) and self.w_up.dtype == torch.bfloat16 and s.intermediate_size % 32 == 0
+                and s.hidden_size % 32 == 0):
+            # a band of 16 rows never holds rows of two experts (nor gate rows beside up rows)
+            self.t_up = ops.tile_weight(self.w_up.view(-1, s.hidden_size))
+            self.t_down = ops.tile_weight(self.w_down.view(-1, s.intermediate_size))
 
     def flops(self, tokens: int) -> float:
         s = self.spec
@@ -91,7 +97,7 @@ class MixtureOfExperts:
         plan = ctx.buffer("moe_plan", (ops.moe_plan_size(n * s.top, s.num_experts, rows),), torch.int32)
         ops.moe_plan(ids, plan, s.num_experts, rows)
         act = ctx.buffer("moe_act", (n * s.top, s.intermediate_size), h.dtype)
-        ops.moe_experts_up(h, self.w_up, plan, act, s.top, s.activation, rows)
+        ops.moe_experts_up(h, self.w_up, plan, act, s.top, s.activation, rows, self.t_up)
         out = ctx.buffer("moe_out", (s.top, n, s.hidden_size), torch.float32)
-        ops.moe_experts_down(act, self.w_down, plan, weights, out, rows)
+        ops.moe_experts_down(act, self.w_down, plan, weights, out, rows, self.t_down)
         return out
