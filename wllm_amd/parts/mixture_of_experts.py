@@ -80,9 +80,10 @@ class MixtureOfExperts:
         return 2.0 * tokens * s.hidden_size * (3 * s.top * s.intermediate_size + s.num_experts)
 
     def bytes_read(self, tokens: int) -> float:
-        """Bytes of expert weights a step of `tokens` tokens reads at most (every chosen expert once)."""
+        """Bytes of expert weights a step of `tokens` tokens reads if the router spreads the tokens evenly: every
+        expert that at least one token chooses, once (experts * (1 - (1 - top / experts) ** tokens) of them)."""
         s = self.spec
-        used = min(s.num_experts, tokens * s.top)
+        used = s.num_experts * (1.0 - (1.0 - s.top / s.num_experts) ** tokens)
         return 3.0 * used * s.intermediate_size * s.hidden_size * self.w_up.element_size()
 
     def forward(self, ctx, h, product_input=None):
