@@ -435,30 +435,29 @@ class EmulatedKernels:
     def moe_plan(self, ids, plan, experts, tile_rows=16):
         self._count("moe_plan")
         flat = ids.reshape(-1).tolist()
-        max_tiles = len(flat) // 16 + experts
-        assert tile_rows == 16, "the emulation plans tiles of 16 rows"
+        max_tiles = len(flat) // tile_rows + experts
         plan.fill_(-7)                       # what the kernels must not read
         tiles = 0
         for e in range(experts):
             mine = [a for a, x in enumerate(flat) if x == e]
-            for t0 in range(0, len(mine), 16):
-                rows = mine[t0:t0 + 16]
+            for t0 in range(0, len(mine), tile_rows):
+                rows = mine[t0:t0 + tile_rows]
                 plan[1 + tiles] = e
-                at = 1 + max_tiles + 16 * tiles
-                plan[at:at + 16] = torch.tensor(rows + [-1] * (16 - len(rows)), dtype=torch.int32)
+                at = 1 + max_tiles + tile_rows * tiles
+                plan[at:at + tile_rows] = torch.tensor(rows + [-1] * (tile_rows - len(rows)), dtype=torch.int32)
                 tiles += 1
         plan[0] = tiles
 
-    def _plan_rows(self, plan, experts, assignments):
-        max_tiles = assignments // 16 + experts
+    def _plan_rows(self, plan, experts, assignments, tile_rows=16):
+        max_tiles = assignments // tile_rows + experts
         for t in range(int(plan[0])):
-            at = 1 + max_tiles + 16 * t
-            yield int(plan[1 + t]), [a for a in plan[at:at + 16].tolist() if a >= 0]
+            at = 1 + max_tiles + tile_rows * t
+            yield int(plan[1 + t]), [a for a in plan[at:at + tile_rows].tolist() if a >= 0]
 
-    def moe_experts_up(self, x, w, plan, act, top, activation, tiles=None):
+    def moe_experts_up(self, x, w, plan, act, top, activation, tiles=None, tile_rows=16):
         self._count("moe_experts_up")
         ff = w.shape[1] // 2
-        for e, rows in self._plan_rows(plan, w.shape[0], act.shape[0]):
+        for e, rows in self._plan_rows(plan, w.shape[0], act.shape[0], tile_rows):
             h = x[[a // top for a in rows]].to(self.acc)
             z, u = h @ w[e, :ff].to(self.acc).T, h @ w[e, ff:].to(self.acc).T
             if activation == "gelu_tanh":
@@ -467,14 +466,22 @@ class EmulatedKernels:
                 z = z * torch.sigmoid(z)
             act[rows] = (z * u).to(act.dtype)
 
-    def moe_experts_down(self, act, w, plan, weights, out, tiles=None):
+    def moe_experts_down(self, act, w, plan, weights, out, tiles=None, tile_rows=16):
         self._count("moe_experts_down")
         n, top = weights.shape
         flat = weights.reshape(-1)
-        for e, rows in self._plan_rows(plan, w.shape[0], act.shape[0]):
+        for e, rows in self._plan_rows(plan, w.shape[0], act.shape[0], tile_rows):
             y = act[rows].to(self.acc) @ w[e].to(self.acc).T
             for a, r in zip(rows, y):
                 out[a % top, a // top] = (r * flat[a].to(self.acc)).float()
+
+    def moe_experts_up_tiled(self, x, w, plan, act, top, activation):
+        self._count("moe_experts_up_tiled")
+        self.moe_experts_up(x, w, plan, act, top, activation, tile_rows=128)
+
+    def moe_experts_down_tiled(self, act, w, plan, weights, out):
+        self._count("moe_experts_down_tiled")
+        self.moe_experts_down(act, w, plan, weights, out, tile_rows=128)
 
     def stream_add(self, x, addend, delta, delta_bias):
         self._count("stream_add")

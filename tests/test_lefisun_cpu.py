@@ -274,3 +274,27 @@ def test_models_of_one_kind_of_mixer(tmp_path, layers):
         got = replay_and_collect(TraceReplayer(runner), trace)
         runner.cache.check()
     compare_rows(got, reference, relative=5e-5)
+
+
+def test_many_rows_an_expert_take_the_plan_of_large_tiles(tmp_path):
+    """bfloat16, sizes in multiples of 64 and a portion of some hundred tokens: the step plans tiles of 128 rows
+    (shorter steps of the same request tiles of 16), and the rows are the plain implementation's within bfloat16."""
+    c = dict(page_size=16, seed=9, config=config(120, 64, [
+        retention(2, 16, 32, (0.9, 0.99), rot(16, 100.0), experts(64, 4, 2, 2, 1)),
+        parallel(left(2, 1, 32, 32, chunk=100, rotation=rot(16, 1000.0)), right(2, 16, 16, 5.0), experts(128, 2, 1), 1.0, 1.0)]))
+    folder = write_folder(c, str(tmp_path / "m"))
+    requests = requests_for(c, [300])
+    reference = plain_logits(folder, requests, torch.float64)
+    toks = requests["q0"]
+    trace = [{"step": 0, "entries": [{"id": "q0", "tokens": toks[:260], "want": list(range(0, 260, 7))}], "end": []},
+             {"step": 1, "entries": [{"id": "q0", "tokens": toks[260:], "want": list(range(40))}], "end": ["q0"]}]
+    with ops.use_backend(EmulatedKernels()) as emulated:
+        model = load_model(folder, "bfloat16", "cpu")
+        runner = ModelRunner.create(model, num_pages=20, page_size=16, max_requests=2)
+        got = replay_and_collect(TraceReplayer(runner), trace)
+        # the first step's two layers took the large tiles, the second step's the small ones
+        assert emulated.calls.get("moe_experts_up_tiled", 0) == 2 and emulated.calls.get("moe_experts_down_tiled", 0) == 2
+        assert emulated.calls.get("moe_experts_up", 0) == 4
+    assert ops.moe_tile_rows(260 * 2, 4, torch.bfloat16, 64, 64) == 128 and ops.moe_tile_rows(40 * 2, 4, torch.bfloat16, 64, 64) == 16
+    assert ops.moe_tile_rows(260 * 2, 4, torch.float32, 64, 64) == 16 and ops.moe_tile_rows(260 * 2, 4, torch.bfloat16, 64, 96) == 16
+    compare_rows(got, reference, relative=0.05, outliers=0.1, ceiling=10.0)

@@ -222,7 +222,9 @@ def test_one_feed_forward_is_added_to_the_stream_it_read_through_a_norm(model_fo
     w = P.read_weights(folder, torch.float64)
     ids = torch.randint(0, cfg["vocab_size"], (7,))
     eps, p = cfg["rms_norm_eps"], "model.layers.0."
-    x = w["model.embed_tokens.weight"][ids] * math.sqrt(cfg["hidden_size"])
+    # (the factor is the reference's float32 buffer, llama.py:397: for a hidden size that is no square its rounding is
+    # 1e-8 of x, which the sum x + mlp keeps where a norm alone would divide it out)
+    x = w["model.embed_tokens.weight"][ids] * float(torch.tensor(cfg["hidden_size"] ** 0.5, dtype=torch.float32))
     h = _hand_norm(x, w[p + "post_attention_layernorm.weight"], eps)
     gate, up = h @ w[p + "mlp.gate_proj.weight"].T, h @ w[p + "mlp.up_proj.weight"].T
     mlp = (torch.nn.functional.gelu(gate, approximate="tanh") * up) @ w[p + "mlp.down_proj.weight"].T
