@@ -295,6 +295,7 @@ def test_many_rows_an_expert_take_the_plan_of_large_tiles(tmp_path):
         # the first step's two layers took the large tiles, the second step's the small ones
         assert emulated.calls.get("moe_experts_up_tiled", 0) == 2 and emulated.calls.get("moe_experts_down_tiled", 0) == 2
         assert emulated.calls.get("moe_experts_up", 0) == 4
-    assert ops.moe_tile_rows(260 * 2, 4, torch.bfloat16, 64, 64) == 128 and ops.moe_tile_rows(40 * 2, 4, torch.bfloat16, 64, 64) == 16
-    assert ops.moe_tile_rows(260 * 2, 4, torch.float32, 64, 64) == 16 and ops.moe_tile_rows(260 * 2, 4, torch.bfloat16, 64, 96) == 16
+    assert ops.moe_tile_rows(260 * 2, 4, torch.bfloat16, 64, 64) == 128 and ops.moe_tile_rows(40 * 2, 4, torch.bfloat16, 64, 64) == 64
+    assert ops.moe_tile_rows(260 * 2, 4, torch.float32, 64, 64) == 64 and ops.moe_tile_rows(260 * 2, 4, torch.bfloat16, 64, 96) == 64
+    assert ops.moe_tile_rows(8, 4, torch.bfloat16, 64, 64) == 16 and ops.moe_tile_rows(48, 4, torch.bfloat16, 64, 64) == 32
     compare_rows(got, reference, relative=0.05, outliers=0.1, ceiling=10.0)

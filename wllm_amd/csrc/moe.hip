@@ -5,7 +5,7 @@
 //            `groups` equal groups of neighbours (a group's score: its largest s) may be chosen; the `top`
 //            allowed experts with the largest s are chosen, weights s / (sum of the chosen + eps)
 //   plan     an assignment is a = token * top + slot.  The assignments of one expert lie together, in
-//            tiles of R rows (16 or 128; the last tile of an expert padded with -1):
+//            tiles of R rows (16, 32, 64 or 128; the last tile of an expert padded with -1):
 //            plan[0] = tiles in use; plan[1 + t] = expert of tile t; plan[1 + max_tiles + R t + r] = a or -1
 //   up       act[a] = activation(x[token] Wg_e^T) * (x[token] Wu_e^T)
 //   down     out[slot][token] = weight[a] * (act[a] Wd_e^T), float32: a stack of `top` partial sums that
@@ -14,6 +14,8 @@
 // not depend on what else the batch holds.  Nothing is read on the host: the grid has room for the most
 // tiles a step of its size can need and a workgroup beyond plan[0] leaves at once.
 #include "common.h"
+
+#include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
@@ -257,14 +259,17 @@ template <> struct MoeFrag<float> {
 };
 
 // act[a, c] = activation(x[token(a)] . Wg[e][c]) * (x[token(a)] . Wu[e][c]); w [experts, 2 * ff, K]: an
-// expert's gate rows, then its up rows.  Grid (tiles, bands of 64 columns); a wavefront 16 columns.
+// expert's gate rows, then its up rows.  Grid (tiles, bands of 64 columns); a wavefront 16 columns.  A tile is MT
+// sub-tiles of 16 rows (the plan's tiles have 16 MT rows): a fragment of the weights feeds MT products, so an expert
+// with up to 16 MT rows reads its weights once.
 // `tiles`: the weights' tile-major copy (bfloat16: per band of 16 rows of the stacked [experts * 2 * ff, K] matrix and
 // step of 32 keys one KiB in lane order, as `wllm_tile_weight` writes it; ff a multiple of 16), or null: then a
 // wavefront's load of a fragment is one contiguous KiB instead of 16 pieces a row apart.
-template <typename T, int ACT>
+template <typename T, int ACT, int MT>
 __global__ void __launch_bounds__(256)
 moe_up_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ tiles, const int* __restrict__ plan,
               int max_tiles, T* __restrict__ act, int K, int ff, int top) {
+    constexpr int U = MT == 4 ? 2 : 4;          // chunks whose loads are asked for before the first product
     const int tile = blockIdx.x;
     if (tile >= plan[0]) return;
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -272,90 +277,108 @@ moe_up_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __restr
     const int c0 = (blockIdx.y * 4 + wave) * 16;
     if (c0 >= ff) return;
     const int e = plan[1 + tile];
-    const int* rows = plan + 1 + max_tiles + tile * kMoeTile;
-    const int a_i = rows[i];
-    const T* xr = x + static_cast<size_t>(a_i >= 0 ? a_i / top : 0) * K;
+    const int* rows = plan + 1 + max_tiles + tile * (kMoeTile * MT);
+    int a_i[MT];
+    const T* xr[MT];
+    float4_t acc_g[MT], acc_u[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        a_i[m] = rows[16 * m + i];
+        xr[m] = x + static_cast<size_t>(a_i[m] >= 0 ? a_i[m] / top : 0) * K;
+        acc_g[m] = acc_u[m] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
     const bool w_live = c0 + i < ff;
     const T* wg = w + (static_cast<size_t>(e) * 2 * ff + (w_live ? c0 + i : 0)) * K;
     const T* wu = wg + static_cast<size_t>(ff) * K;
-    float4_t acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
     constexpr int kChunk = MoeFrag<T>::kChunk, kPer = MoeFrag<T>::kPer;
-    if (tiles != nullptr && K % (4 * kChunk) == 0) {
+    if (K % (4 * kChunk) == 0) {
+        // every fragment is whole (rows that stand for nothing read row 0, and their sums are dropped)
+        const bool tiled = tiles != nullptr;
         const size_t per_band = static_cast<size_t>(K / kChunk) * kWave * kPer;        // elements of a band's tiles
-        const T* tg = tiles + (static_cast<size_t>(e) * 2 * ff + c0) / 16 * per_band + lane * kPer;
-        const T* tu = tiles + (static_cast<size_t>(e) * 2 * ff + ff + c0) / 16 * per_band + lane * kPer;
-        for (int k0 = 0; k0 < K; k0 += 4 * kChunk) {
-            MoeFrag<T> fx[4], fg[4], fu[4];
+        const T* tg = tiled ? tiles + (static_cast<size_t>(e) * 2 * ff + c0) / 16 * per_band + lane * kPer : wg + g * kPer;
+        const T* tu = tiled ? tiles + (static_cast<size_t>(e) * 2 * ff + ff + c0) / 16 * per_band + lane * kPer : wu + g * kPer;
+        // (the step from a chunk's fragment to the next chunk's is a constant either way, so that the loads of a
+        // round differ by immediate offsets)
+        auto walk = [&](auto step) {
+            constexpr int kStep = decltype(step)::value;
+            for (int k0 = 0; k0 < K; k0 += U * kChunk) {
+                MoeFrag<T> fx[U][MT], fg[U], fu[U];
+                const T* pg = tg + static_cast<size_t>(k0 / kChunk) * kStep;
+                const T* pu = tu + static_cast<size_t>(k0 / kChunk) * kStep;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                fx[u].whole(xr + k0 + u * kChunk + g * kPer);
-                fg[u].template whole<true>(tg + static_cast<size_t>(k0 / kChunk + u) * kWave * kPer);
-                fu[u].template whole<true>(tu + static_cast<size_t>(k0 / kChunk + u) * kWave * kPer);
-            }
+                for (int u = 0; u < U; ++u) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                acc_g = MoeFrag<T>::mma(fg[u], fx[u], acc_g);
-                acc_u = MoeFrag<T>::mma(fu[u], fx[u], acc_u);
-            }
-        }
-    } else if (K % (4 * kChunk) == 0) {
-        // every fragment is whole (rows that stand for nothing read row 0, and their sums are dropped); four
-        // chunks' loads are asked for before the first product
-        for (int k0 = g * kPer; k0 < K; k0 += 4 * kChunk) {
-            MoeFrag<T> fx[4], fg[4], fu[4];
+                    for (int m = 0; m < MT; ++m) fx[u][m].whole(xr[m] + k0 + u * kChunk + g * kPer);
+                    fg[u].template whole<true>(pg + u * kStep);
+                    fu[u].template whole<true>(pu + u * kStep);
+                }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                fx[u].whole(xr + k0 + u * kChunk);
-                fg[u].template whole<true>(wg + k0 + u * kChunk);
-                fu[u].template whole<true>(wu + k0 + u * kChunk);
-            }
+                for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                acc_g = MoeFrag<T>::mma(fg[u], fx[u], acc_g);
-                acc_u = MoeFrag<T>::mma(fu[u], fx[u], acc_u);
+                    for (int m = 0; m < MT; ++m) {
+                        acc_g[m] = MoeFrag<T>::mma(fg[u], fx[u][m], acc_g[m]);
+                        acc_u[m] = MoeFrag<T>::mma(fu[u], fx[u][m], acc_u[m]);
+                    }
             }
-        }
+        };
+        if (tiled) walk(std::integral_constant<int, kWave * kPer>{});
+        else walk(std::integral_constant<int, kChunk>{});
     } else {
         for (int k0 = 0; k0 < K; k0 += kChunk) {
-            MoeFrag<T> fx, fg, fu;
+            MoeFrag<T> fg, fu;
             const int k = k0 + g * kPer;
-            fx.load(xr, k, K, a_i >= 0);
             fg.load(wg, k, K, w_live);
             fu.load(wu, k, K, w_live);
-            acc_g = MoeFrag<T>::mma(fg, fx, acc_g);
-            acc_u = MoeFrag<T>::mma(fu, fx, acc_u);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                MoeFrag<T> fx;
+                fx.load(xr[m], k, K, a_i[m] >= 0);
+                acc_g[m] = MoeFrag<T>::mma(fg, fx, acc_g[m]);
+                acc_u[m] = MoeFrag<T>::mma(fu, fx, acc_u[m]);
+            }
         }
     }
-    if (a_i < 0) return;
-    T* out = act + static_cast<size_t>(a_i) * ff;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const int c = c0 + 4 * g + v;
-        if (c < ff) out[c] = from_float<T>(activate<ACT>(acc_g[v]) * acc_u[v]);
+    for (int m = 0; m < MT; ++m) {
+        if (a_i[m] < 0) continue;
+        T* out = act + static_cast<size_t>(a_i[m]) * ff;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int c = c0 + 4 * g + v;
+            if (c < ff) out[c] = from_float<T>(activate<ACT>(acc_g[m][v]) * acc_u[m][v]);
+        }
     }
 }
 
-WLLM_API int wllm_moe_up(const void* x, const void* w, const void* tiles, const int* plan, int max_tiles, void* act, int is_bf16,
-                         int activation, int K, int ff, int top, hipStream_t stream) {
+// `tile_rows`: the rows of the plan's tiles, 16, 32 or 64.
+WLLM_API int wllm_moe_up(const void* x, const void* w, const void* tiles, const int* plan, int max_tiles, int tile_rows,
+                         void* act, int is_bf16, int activation, int K, int ff, int top, hipStream_t stream) {
     if (max_tiles <= 0) return 0;
     if (K <= 0 || ff <= 0 || top <= 0 || activation < 0 || activation >= kActivations || (ff + 63) / 64 > 65535) return -1;
+    if (tile_rows != 16 && tile_rows != 32 && tile_rows != 64) return -1;
     if (tiles && (!is_bf16 || ff % 16 || K % 32)) return -1;
     const dim3 grid(max_tiles, (ff + 63) / 64);
-#define LAUNCH(T)                                                                                                     \
-    WLLM_BY_ACTIVATION(activation, (moe_up_kernel<T, ACT><<<grid, 256, 0, stream>>>(                                  \
+#define LAUNCH_MT(T, MT)                                                                                              \
+    WLLM_BY_ACTIVATION(activation, (moe_up_kernel<T, ACT, MT><<<grid, 256, 0, stream>>>(                              \
                                        static_cast<const T*>(x), static_cast<const T*>(w), static_cast<const T*>(tiles), \
                                        plan, max_tiles, static_cast<T*>(act), K, ff, top)))
-    if (is_bf16) { LAUNCH(bf16); } else { LAUNCH(float); }
+#define LAUNCH(T)                                    \
+    if (tile_rows == 16) { LAUNCH_MT(T, 1); }        \
+    else if (tile_rows == 32) { LAUNCH_MT(T, 2); }   \
+    else { LAUNCH_MT(T, 4); }
+    if (is_bf16) { LAUNCH(bf16) } else { LAUNCH(float) }
 #undef LAUNCH
+#undef LAUNCH_MT
     return launch_status();
 }
 
 // out[a % top][a / top][c] = weight[a] * (act[a] . Wd[e][c]); w [experts, width, ff]; out float32 [top, tokens, width].
-template <typename T>
+template <typename T, int MT>
 __global__ void __launch_bounds__(256)
 moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w, const T* __restrict__ tiles, const int* __restrict__ plan,
                 int max_tiles, const float* __restrict__ weights, float* __restrict__ out, int tokens, int ff, int width,
                 int top) {
+    constexpr int U = 4;
     const int tile = blockIdx.x;
     if (tile >= plan[0]) return;
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -363,70 +386,87 @@ moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w, const T* __r
     const int c0 = (blockIdx.y * 4 + wave) * 16;
     if (c0 >= width) return;
     const int e = plan[1 + tile];
-    const int* rows = plan + 1 + max_tiles + tile * kMoeTile;
-    const int a_i = rows[i];
-    const T* xr = act + static_cast<size_t>(a_i >= 0 ? a_i : 0) * ff;
+    const int* rows = plan + 1 + max_tiles + tile * (kMoeTile * MT);
+    int a_i[MT];
+    const T* xr[MT];
+    float4_t acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        a_i[m] = rows[16 * m + i];
+        xr[m] = act + static_cast<size_t>(a_i[m] >= 0 ? a_i[m] : 0) * ff;
+        acc[m] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
     const bool w_live = c0 + i < width;
     const T* wd = w + (static_cast<size_t>(e) * width + (w_live ? c0 + i : 0)) * ff;
-    float4_t acc = {0.f, 0.f, 0.f, 0.f};
     constexpr int kChunk = MoeFrag<T>::kChunk, kPer = MoeFrag<T>::kPer;
-    if (tiles != nullptr && ff % (4 * kChunk) == 0) {
+    if (ff % (4 * kChunk) == 0) {
+        const bool tiled = tiles != nullptr;
         const size_t per_band = static_cast<size_t>(ff / kChunk) * kWave * kPer;
-        const T* td = tiles + (static_cast<size_t>(e) * width + c0) / 16 * per_band + lane * kPer;
-        for (int k0 = 0; k0 < ff; k0 += 4 * kChunk) {
-            MoeFrag<T> fx[4], fw[4];
+        const T* td = tiled ? tiles + (static_cast<size_t>(e) * width + c0) / 16 * per_band + lane * kPer : wd + g * kPer;
+        auto walk = [&](auto step) {
+            constexpr int kStep = decltype(step)::value;
+            for (int k0 = 0; k0 < ff; k0 += U * kChunk) {
+                MoeFrag<T> fx[U][MT], fw[U];
+                const T* pd = td + static_cast<size_t>(k0 / kChunk) * kStep;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                fx[u].whole(xr + k0 + u * kChunk + g * kPer);
-                fw[u].template whole<true>(td + static_cast<size_t>(k0 / kChunk + u) * kWave * kPer);
+                for (int u = 0; u < U; ++u) {
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) fx[u][m].whole(xr[m] + k0 + u * kChunk + g * kPer);
+                    fw[u].template whole<true>(pd + u * kStep);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) acc[m] = MoeFrag<T>::mma(fw[u], fx[u][m], acc[m]);
             }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) acc = MoeFrag<T>::mma(fw[u], fx[u], acc);
-        }
-    } else if (ff % (4 * kChunk) == 0) {
-        for (int k0 = g * kPer; k0 < ff; k0 += 4 * kChunk) {
-            MoeFrag<T> fx[4], fw[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                fx[u].whole(xr + k0 + u * kChunk);
-                fw[u].template whole<true>(wd + k0 + u * kChunk);
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) acc = MoeFrag<T>::mma(fw[u], fx[u], acc);
-        }
+        };
+        if (tiled) walk(std::integral_constant<int, kWave * kPer>{});
+        else walk(std::integral_constant<int, kChunk>{});
     } else {
         for (int k0 = 0; k0 < ff; k0 += kChunk) {
-            MoeFrag<T> fx, fw;
+            MoeFrag<T> fw;
             const int k = k0 + g * kPer;
-            fx.load(xr, k, ff, a_i >= 0);
             fw.load(wd, k, ff, w_live);
-            acc = MoeFrag<T>::mma(fw, fx, acc);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                MoeFrag<T> fx;
+                fx.load(xr[m], k, ff, a_i[m] >= 0);
+                acc[m] = MoeFrag<T>::mma(fw, fx, acc[m]);
+            }
         }
     }
-    if (a_i < 0) return;
-    const float weight = weights[a_i];
-    float* o = out + (static_cast<size_t>(a_i % top) * tokens + a_i / top) * width;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const int c = c0 + 4 * g + v;
-        if (c < width) o[c] = weight * acc[v];
+    for (int m = 0; m < MT; ++m) {
+        if (a_i[m] < 0) continue;
+        const float weight = weights[a_i[m]];
+        float* o = out + (static_cast<size_t>(a_i[m] % top) * tokens + a_i[m] / top) * width;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int c = c0 + 4 * g + v;
+            if (c < width) o[c] = weight * acc[m][v];
+        }
     }
 }
 
-WLLM_API int wllm_moe_down(const void* act, const void* w, const void* tiles, const int* plan, int max_tiles,
+WLLM_API int wllm_moe_down(const void* act, const void* w, const void* tiles, const int* plan, int max_tiles, int tile_rows,
                            const float* weights, float* out, int is_bf16, int tokens, int ff, int width, int top,
                            hipStream_t stream) {
     if (max_tiles <= 0 || tokens <= 0) return 0;
     if (ff <= 0 || width <= 0 || top <= 0 || (width + 63) / 64 > 65535) return -1;
+    if (tile_rows != 16 && tile_rows != 32 && tile_rows != 64) return -1;
     if (tiles && (!is_bf16 || width % 16 || ff % 32)) return -1;
     const dim3 grid(max_tiles, (width + 63) / 64);
-    if (is_bf16)
-        moe_down_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(act), static_cast<const bf16*>(w),
-                                                        static_cast<const bf16*>(tiles), plan, max_tiles, weights, out, tokens,
-                                                        ff, width, top);
-    else
-        moe_down_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(act), static_cast<const float*>(w), nullptr,
-                                                         plan, max_tiles, weights, out, tokens, ff, width, top);
+#define LAUNCH_MT(T, MT)                                                                                              \
+    moe_down_kernel<T, MT><<<grid, 256, 0, stream>>>(static_cast<const T*>(act), static_cast<const T*>(w),             \
+                                                     static_cast<const T*>(tiles), plan, max_tiles, weights, out, tokens, \
+                                                     ff, width, top)
+#define LAUNCH(T)                                    \
+    if (tile_rows == 16) LAUNCH_MT(T, 1);            \
+    else if (tile_rows == 32) LAUNCH_MT(T, 2);       \
+    else LAUNCH_MT(T, 4);
+    if (is_bf16) { LAUNCH(bf16) } else { LAUNCH(float) }
+#undef LAUNCH
+#undef LAUNCH_MT
     return launch_status();
 }
 

@@ -1002,16 +1002,22 @@ def head_norm_gate(y: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.T
 
 
 # ---- a mixture of experts ------------------------------------------------------------------------------
-MOE_TILE_ROWS = 16           # rows of a tile of the kernels that stream an expert's weights past a few rows
+MOE_TILE_ROWS = 16           # rows of a tile of the kernels that stream an expert's weights past a few rows: 16, 32 or 64
+MOE_STREAM_TILE_ROWS = (16, 32, 64)
 MOE_BIG_TILE_ROWS = 128      # rows of a tile of the kernel that tiles many rows an expert through shared memory
 MOE_MAX_EXPERTS = 256
 
 
 def moe_tile_rows(assignments: int, experts: int, dtype, *inner_sizes: int) -> int:
     """The tile a step's plan should have: tiles of 128 rows where the experts get some tens of rows each on average
-    (a prompt's portion) and the tiled kernel takes the sizes (bfloat16, inner sizes in multiples of 64), else 16."""
+    (a prompt's portion) and the tiled kernel takes the sizes (bfloat16, inner sizes in multiples of 64); else tiles of
+    16, 32 or 64 rows for the kernels that stream the weights (a fragment of the weights feeds a product for every 16
+    rows of the tile): the smallest that most experts fill no more than once, so that their weights are read once."""
     big = dtype == torch.bfloat16 and assignments >= 32 * experts and all(k % 64 == 0 and k >= 64 for k in inner_sizes)
-    return MOE_BIG_TILE_ROWS if big else MOE_TILE_ROWS
+    if big:
+        return MOE_BIG_TILE_ROWS
+    mean = assignments / experts
+    return 16 if mean <= 6 else 32 if mean <= 16 else 64
 
 
 def moe_max_tiles(assignments: int, experts: int, tile_rows: int = MOE_TILE_ROWS) -> int:
@@ -1058,14 +1064,14 @@ def moe_plan(ids: torch.Tensor, plan: torch.Tensor, experts: int, tile_rows: int
     _dense(ids, "ids", torch.int32)
     _need(ids.dim() == 2, "ids: expected [n, top]")
     _need(0 < experts <= MOE_MAX_EXPERTS, f"experts: from 1 to {MOE_MAX_EXPERTS}")
-    _need(tile_rows in (MOE_TILE_ROWS, MOE_BIG_TILE_ROWS), "tile_rows: 16 or 128")
+    _need(tile_rows in MOE_STREAM_TILE_ROWS or tile_rows == MOE_BIG_TILE_ROWS, "tile_rows: 16, 32, 64 or 128")
     _dense(plan, "plan", torch.int32, (moe_plan_size(ids.numel(), experts, tile_rows),))
     if ids.numel():
         call("moe_plan", ids, plan, int(experts), int(tile_rows))
 
 
 def _big_tiles(tile_rows: int, dtype, inner: int) -> bool:
-    _need(tile_rows in (MOE_TILE_ROWS, MOE_BIG_TILE_ROWS), "tile_rows: 16 or 128")
+    _need(tile_rows in MOE_STREAM_TILE_ROWS or tile_rows == MOE_BIG_TILE_ROWS, "tile_rows: 16, 32, 64 or 128")
     if tile_rows == MOE_BIG_TILE_ROWS:
         _need(dtype == torch.bfloat16 and inner % 64 == 0 and inner >= 64,
               "tiles of 128 rows: bfloat16 and an inner size that is a multiple of 64")
@@ -1101,7 +1107,7 @@ def moe_experts_up(x: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, act: to
         if _big_tiles(tile_rows, x.dtype, width):
             call("moe_experts_up_tiled", x, w, plan, act, int(top), activation)
         else:
-            call("moe_experts_up", x, w, plan, act, int(top), activation, tiles)
+            call("moe_experts_up", x, w, plan, act, int(top), activation, tiles, int(tile_rows))
 
 
 def moe_experts_down(act: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, weights: torch.Tensor,
@@ -1123,7 +1129,7 @@ def moe_experts_down(act: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, wei
         if _big_tiles(tile_rows, act.dtype, act.shape[1]):
             call("moe_experts_down_tiled", act, w, plan, weights, out)
         else:
-            call("moe_experts_down", act, w, plan, weights, out, tiles)
+            call("moe_experts_down", act, w, plan, weights, out, tiles, int(tile_rows))
 
 
 # ---- the framework's own operations that go through the same door as a part's ------------------
@@ -1285,16 +1291,17 @@ def _register_own() -> None:
                 launch=lambda fn, stream, ids, plan, experts, tile_rows=MOE_TILE_ROWS: fn(
                     p(ids), p(plan), ids.numel(), experts, moe_max_tiles(ids.numel(), experts, tile_rows), tile_rows, stream))
     register_op("moe_experts_up", entry_point="wllm_moe_up",
-                argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
-                launch=lambda fn, stream, x, w, plan, act, top, activation, tiles=None: fn(
-                    p(x), p(w), p(tiles), p(plan), moe_max_tiles(act.shape[0], w.shape[0]), p(act), bf(x),
+                argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                          c_void_p],
+                launch=lambda fn, stream, x, w, plan, act, top, activation, tiles=None, tile_rows=MOE_TILE_ROWS: fn(
+                    p(x), p(w), p(tiles), p(plan), moe_max_tiles(act.shape[0], w.shape[0], tile_rows), tile_rows, p(act), bf(x),
                     ACTIVATIONS[activation], x.shape[1], act.shape[1], top, stream))
     register_op("moe_experts_down", entry_point="wllm_moe_down",
-                argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                          c_void_p],
-                launch=lambda fn, stream, act, w, plan, weights, out, tiles=None: fn(
-                    p(act), p(w), p(tiles), p(plan), moe_max_tiles(act.shape[0], w.shape[0]), p(weights), p(out), bf(act),
-                    weights.shape[0], act.shape[1], w.shape[1], weights.shape[1], stream))
+                argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                          c_int, c_void_p],
+                launch=lambda fn, stream, act, w, plan, weights, out, tiles=None, tile_rows=MOE_TILE_ROWS: fn(
+                    p(act), p(w), p(tiles), p(plan), moe_max_tiles(act.shape[0], w.shape[0], tile_rows), tile_rows, p(weights),
+                    p(out), bf(act), weights.shape[0], act.shape[1], w.shape[1], weights.shape[1], stream))
     tiles = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
              c_void_p]
     register_op("moe_experts_up_tiled", entry_point="wllm_moe_tiles", argtypes=tiles,

@@ -8,9 +8,9 @@
 The experts' matrices are stacked at load ([experts, 2 * ff, width]: an expert's gate rows, then its up
 rows; [experts, width, ff]).  A step routes its tokens, sorts the (token, expert) pairs by expert on the
 device (`ops.moe_plan`: tiles of rows of one expert) and runs the two products expert by expert on
-the matrix cores, each tile with its expert's weights: tiles of 16 rows past which an expert's weights
-stream where the experts get few rows each (decoded tokens), tiles of 128 rows through shared memory
-where they get many (a prompt's portion).  The second product weighs a pair's result and
+the matrix cores, each tile with its expert's weights: tiles of 16 to 64 rows past which an expert's
+weights stream where the experts get few rows each (decoded tokens), tiles of 128 rows through shared
+memory where they get many (a prompt's portion).  The second product weighs a pair's result and
 leaves it in the slice of its slot of a float32 stack [top, tokens, width], which whoever adds the
 feed-forward to the stream (the next norm kernel) adds in order: the weighted sum is formed in float32
 and takes no pass of its own.  Nothing of the routing is read on the host.
