@@ -179,7 +179,7 @@ class EmulatedKernels:
         return None
 
     def head_prepare(self, rows, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim, page_size,
-                     interleaved, norm_eps, values_are_keys, parts, norm_dim=None):
+                     interleaved, norm_eps, values_are_keys, parts, norm_dim=None, head_norm=None, rot_scale=1.0):
         self._count("head_prepare")
         n, width = rows.shape
         if parts is not None:
@@ -195,10 +195,15 @@ class EmulatedKernels:
         r = num_heads + num_kv_heads
         heads = v[:, :r * head_dim].reshape(n, r, head_dim).clone()
         as_projected = heads[:, num_heads:].clone()
+        if head_norm is not None:
+            w_q, w_k, pre_eps = head_norm
+            heads = heads * torch.rsqrt(heads.pow(2).sum(-1, keepdim=True) / (norm_dim or head_dim) + pre_eps)
+            heads[:, :num_heads] *= w_q.to(self.acc)
+            heads[:, num_heads:] *= w_k.to(self.acc)
         if inv_freq is not None:
             half = inv_freq.shape[0]
             ang = positions.to(torch.float32)[:, None] * inv_freq[None, :]          # float32 angles
-            cos, sin = ang.cos().to(self.acc)[:, None, :], ang.sin().to(self.acc)[:, None, :]
+            cos, sin = (ang.cos() * rot_scale).to(self.acc)[:, None, :], (ang.sin() * rot_scale).to(self.acc)[:, None, :]
             if interleaved:
                 x1, x2 = heads[..., 0:2 * half:2].clone(), heads[..., 1:2 * half:2].clone()
                 heads[..., 0:2 * half:2] = x1 * cos - x2 * sin
@@ -301,6 +306,22 @@ class EmulatedKernels:
             if taps > 1:
                 carried.copy_(seq[ql:].to(torch.float32))
 
+    def stream_conv(self, x, weight, state, carried_offset, token_segment, seg_q_start, seg_q_len, state_slots, out):
+        self._count("stream_conv")
+        c, taps = weight.shape
+        for s in range(seg_q_start.shape[0]):
+            q0, ql, slot = int(seg_q_start[s]), int(seg_q_len[s]), int(state_slots[s])
+            if ql == 0:
+                continue
+            carried = state[slot, carried_offset:carried_offset + (taps - 1) * c].view(taps - 1, c)
+            seq = torch.cat([carried.to(self.acc), x[q0:q0 + ql].to(self.acc)], dim=0)
+            acc = x[q0:q0 + ql].to(self.acc).clone()
+            for k in range(taps):
+                acc = acc + seq[k:k + ql] * weight[:, k].to(self.acc)
+            out[q0:q0 + ql] = acc.to(out.dtype)
+            if taps > 1:
+                carried.copy_(seq[ql:ql + taps - 1].float())
+
     def ssm_scan(self, xbc, dt, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, state_slots, y, heads, groups,
                  state_size, head_dim, steps=None):
         self._count("ssm_scan")
@@ -352,6 +373,18 @@ class EmulatedKernels:
         qk[0].copy_((v[:, 0] * q_scale).to(torch.float32))
         qk[1].copy_((v[:, 1] * k_scale).to(torch.float32))
 
+    def memory_forget_inputs(self, row, bias, lower, qkf, width, q_activation):
+        self._count("memory_forget_inputs")
+        acc = self.acc
+        q, z = row[:, :width].to(acc), row[:, width:2 * width].to(acc)
+        if bias is not None:
+            z = z + bias.to(acc)
+        low = lower.to(acc) if lower is not None else torch.zeros(width, dtype=acc)
+        f = low + (1.0 - low) * torch.sigmoid(z)
+        qkf[0].copy_((q * torch.sigmoid(q) if q_activation == "silu" else q).float())
+        qkf[1].copy_((1.0 - f).float())
+        qkf[2].copy_(f.float())
+
     def memory_gates(self, gates, i_bias, f_bias, state, m_offset, seg_q_start, seg_q_len, state_slots, steps, heads, cap):
         self._count("memory_gates")
         acc = self.acc
@@ -376,7 +409,7 @@ class EmulatedKernels:
             state[slot, m_offset:m_offset + heads] = m.float()
 
     def memory_scan(self, qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads, head_dim, value_dim,
-                    nq=None, n_offset=0):
+                    nq=None, n_offset=0, row_decays=False):
         self._count("memory_scan")
         acc = self.acc
         size, width = heads * head_dim * value_dim, heads * head_dim
@@ -391,9 +424,12 @@ class EmulatedKernels:
                     a, b = steps[0, t].to(acc), steps[1, t].to(acc)
                     nv = a[:, None] * nv + b[:, None] * k
                     nq[t] = (nv * q).sum(-1).float()
+                elif row_decays:
+                    a, b = None, torch.ones(heads, dtype=acc)
+                    S = qk[2, t].to(acc).view(heads, head_dim)[:, :, None] * S
                 else:
                     a, b = decays.to(acc), torch.ones(heads, dtype=acc)
-                S = a[:, None, None] * S + (b[:, None] * k)[:, :, None] * val[:, None, :]
+                S = (1.0 if a is None else a[:, None, None]) * S + (b[:, None] * k)[:, :, None] * val[:, None, :]
                 y[t] = torch.einsum("hdv,hd->hv", S, q).reshape(-1).float()
             state[slot, :size] = S.reshape(-1).float()
             if steps is not None:
@@ -408,15 +444,17 @@ class EmulatedKernels:
         v = (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)).reshape(n, w)
         if weight is not None:
             v = v * weight.to(self.acc)
-        z = gate.to(self.acc)
-        act = torch.sigmoid(z) if activation == "sigmoid" else z * torch.sigmoid(z)
-        out.copy_((v * act * scale).to(out.dtype))
+        if activation != "none":
+            z = gate.to(self.acc)
+            v = v * (torch.sigmoid(z) if activation == "sigmoid" else z * torch.sigmoid(z))
+        out.copy_((v * scale).to(out.dtype))
 
     # ---- a mixture of experts ---------------------------------------------------------------------
-    def moe_route(self, x, router, ids, weights, groups, keep, eps):
+    def moe_route(self, x, router, ids, weights, groups, keep, eps, scoring="softmax", normalize=True):
         self._count("moe_route")
         n, experts, top = x.shape[0], router.shape[0], ids.shape[1]
-        s = torch.softmax(x.to(self.acc) @ router.to(self.acc).T, dim=-1)
+        z = x.to(self.acc) @ router.to(self.acc).T
+        s = torch.sigmoid(z) if scoring == "sigmoid" else torch.softmax(z, dim=-1)
         allowed = torch.ones(n, experts, dtype=torch.bool)
         if keep < groups:
             per = experts // groups
@@ -430,7 +468,7 @@ class EmulatedKernels:
             order = sorted([e for e in range(experts) if allowed[r, e]], key=lambda e: (-float(s[r, e]), e))[:top]
             chosen = s[r, order]
             ids[r] = torch.tensor(order, dtype=torch.int32)
-            weights[r] = (chosen / (chosen.sum() + eps)).float()
+            weights[r] = (chosen / (chosen.sum() + eps) if normalize else chosen).float()
 
     def moe_plan(self, ids, plan, experts, tile_rows=16):
         self._count("moe_plan")
@@ -454,34 +492,37 @@ class EmulatedKernels:
             at = 1 + max_tiles + tile_rows * t
             yield int(plan[1 + t]), [a for a in plan[at:at + tile_rows].tolist() if a >= 0]
 
-    def moe_experts_up(self, x, w, plan, act, top, activation, tiles=None, tile_rows=16):
+    def moe_experts_up(self, x, w, plan, act, top, activation, tiles=None, tile_rows=16, in_weights=None):
         self._count("moe_experts_up")
         ff = w.shape[1] // 2
         for e, rows in self._plan_rows(plan, w.shape[0], act.shape[0], tile_rows):
             h = x[[a // top for a in rows]].to(self.acc)
             z, u = h @ w[e, :ff].to(self.acc).T, h @ w[e, ff:].to(self.acc).T
+            if in_weights is not None:
+                factor = in_weights.reshape(-1)[rows].to(self.acc)[:, None]
+                z, u = z * factor, u * factor
             if activation == "gelu_tanh":
                 z = 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
             else:
                 z = z * torch.sigmoid(z)
             act[rows] = (z * u).to(act.dtype)
 
-    def moe_experts_down(self, act, w, plan, weights, out, tiles=None, tile_rows=16):
+    def moe_experts_down(self, act, w, plan, weights, out, tiles=None, tile_rows=16, weighted=True):
         self._count("moe_experts_down")
         n, top = weights.shape
-        flat = weights.reshape(-1)
+        flat = weights.reshape(-1) if weighted else torch.ones(weights.numel())
         for e, rows in self._plan_rows(plan, w.shape[0], act.shape[0], tile_rows):
             y = act[rows].to(self.acc) @ w[e].to(self.acc).T
             for a, r in zip(rows, y):
                 out[a % top, a // top] = (r * flat[a].to(self.acc)).float()
 
-    def moe_experts_up_tiled(self, x, w, plan, act, top, activation):
+    def moe_experts_up_tiled(self, x, w, plan, act, top, activation, in_weights=None):
         self._count("moe_experts_up_tiled")
-        self.moe_experts_up(x, w, plan, act, top, activation, tile_rows=128)
+        self.moe_experts_up(x, w, plan, act, top, activation, tile_rows=128, in_weights=in_weights)
 
-    def moe_experts_down_tiled(self, act, w, plan, weights, out):
+    def moe_experts_down_tiled(self, act, w, plan, weights, out, weighted=True):
         self._count("moe_experts_down_tiled")
-        self.moe_experts_down(act, w, plan, weights, out, tile_rows=128)
+        self.moe_experts_down(act, w, plan, weights, out, tile_rows=128, weighted=weighted)
 
     def stream_add(self, x, addend, delta, delta_bias):
         self._count("stream_add")

@@ -19,8 +19,11 @@ template <typename T> struct alignas(4 * sizeof(T)) Four { T v[4]; };
 //   1. the element is the row's (or the sum of the stack of partial sums `parts`), plus its bias
 //      (the bias covers the row's first bias_width columns);
 //   2. where the values are the keys, the key head as it is now goes to the cache's values;
+//   2b. with pre_eps >= 0 the head is divided by sqrt(sum of its squares / norm_dim + pre_eps) and multiplied
+//      element by element by a weight of head_dim numbers (pre_q for query heads, pre_k for key heads): an RMS
+//      norm with a weight over each head, in front of the rotation;
 //   3. the first rotary_dim elements turn by position * inv_freq[j]: pair j is (2j, 2j + 1)
-//      (interleaved) or (j, j + rotary_dim / 2);
+//      (interleaved) or (j, j + rotary_dim / 2); sine and cosine are multiplied by rot_scale;
 //   4. with norm_eps >= 0 the head is divided by sqrt(sum of its squares / norm_dim + norm_eps) (norm_dim is
 //      head_dim, or less where the last elements of a head are padding that is always zero);
 //   5. it is written back to the row, and a key head to the cache's keys.
@@ -40,7 +43,8 @@ head_prepare_kernel(T* __restrict__ rows, int row_width, const float* __restrict
                     const float* __restrict__ bias, int bias_width, const int* __restrict__ positions,
                     const float* __restrict__ inv_freq, const int* __restrict__ slots, T* __restrict__ cache,
                     long long num_pages, int num_heads, int num_kv_heads, int head_dim, int rotary_dim,
-                    int interleaved, float norm_eps, int norm_dim, int values_are_keys, int page_size, int head_pieces) {
+                    int interleaved, float norm_eps, int norm_dim, int values_are_keys, int page_size, int head_pieces,
+                    const float* __restrict__ pre_q, const float* __restrict__ pre_k, float pre_eps, float rot_scale) {
     __shared__ float staged[kPrepareWaves][FOUR ? 1 : kPrepareMaxHead];
     const int token = blockIdx.x;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -128,13 +132,25 @@ head_prepare_kernel(T* __restrict__ rows, int row_width, const float* __restrict
                 for (int u = 0; u < 4; ++u)
                     vpage[(static_cast<size_t>(kvh) * head_dim + e + u) * page_size + off] = from_float<T>(v[u]);
             }
+        }
+        if (pre_eps >= 0.f) {
+            // (every lane of the wavefront takes part in the sum; lanes beyond the head hold zeros)
+            const float ss = wave_sum(v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3]);
+            const float pre = rsqrtf(ss / static_cast<float>(norm_dim) + pre_eps);
+            if (live) {
+                const float* pw = (kvh >= 0 ? pre_k : pre_q) + e;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = v[u] * pre * pw[u];
+            }
+        }
+        if (live) {
             if (inv_freq) {
 #pragma unroll
                 for (int u = 0; u < 4; u += 2) {
                     if (e + u < rotary_dim) {
                         float sn, cs, ra, rb;
                         sincosf(pos * inv_freq[(e + u) >> 1], &sn, &cs);
-                        rotate_pair(v[u], v[u + 1], sn, cs, ra, rb);
+                        rotate_pair(v[u], v[u + 1], sn * rot_scale, cs * rot_scale, ra, rb);
                         v[u] = ra;
                         v[u + 1] = rb;
                     }
@@ -163,9 +179,25 @@ head_prepare_kernel(T* __restrict__ rows, int row_width, const float* __restrict
     for (int k = 0; k < kPerLane; ++k) {
         const int e = lane + k * kWave;
         v[k] = e < head_dim ? value(base + e) : 0.f;
-        if (e < head_dim) mine[e] = v[k];
         if (values_are_keys && kvh >= 0 && vpage && e < head_dim)
             vpage[(static_cast<size_t>(kvh) * head_dim + e) * page_size + off] = from_float<T>(v[k]);
+    }
+    if (pre_eps >= 0.f) {
+        float pss = 0.f;
+#pragma unroll
+        for (int k = 0; k < kPerLane; ++k) pss += v[k] * v[k];
+        const float pre = rsqrtf(wave_sum(pss) / static_cast<float>(norm_dim) + pre_eps);
+        const float* pw = kvh >= 0 ? pre_k : pre_q;
+#pragma unroll
+        for (int k = 0; k < kPerLane; ++k) {
+            const int e = lane + k * kWave;
+            if (e < head_dim) v[k] = v[k] * pre * pw[e];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) {
+        const int e = lane + k * kWave;
+        if (e < head_dim) mine[e] = v[k];
     }
     // lanes read below what other lanes of the wavefront wrote above
     __builtin_amdgcn_wave_barrier();
@@ -181,7 +213,7 @@ head_prepare_kernel(T* __restrict__ rows, int row_width, const float* __restrict
             const float other = mine[partner];
             float sn, cs, ra, rb;
             sincosf(pos * inv_freq[j], &sn, &cs);
-            rotate_pair(first ? v[k] : other, first ? other : v[k], sn, cs, ra, rb);
+            rotate_pair(first ? v[k] : other, first ? other : v[k], sn * rot_scale, cs * rot_scale, ra, rb);
             v[k] = first ? ra : rb;
         }
         ss += v[k] * v[k];
@@ -205,7 +237,9 @@ WLLM_API int wllm_head_prepare(void* rows, int is_bf16, int row_width, const flo
                                long long split_stride, const float* bias, int bias_width, const int* positions,
                                const float* inv_freq, const int* slots, void* cache, long long num_pages, int n,
                                int num_heads, int num_kv_heads, int head_dim, int rotary_dim, int interleaved,
-                               float norm_eps, int norm_dim, int values_are_keys, int page_size, hipStream_t stream) {
+                               float norm_eps, int norm_dim, int values_are_keys, int page_size, const float* pre_q,
+                               const float* pre_k, float pre_eps, float rot_scale, hipStream_t stream) {
+    if (pre_eps >= 0.f && (pre_q == nullptr || (pre_k == nullptr && num_kv_heads > 0))) return -1;
     const int heads = num_heads + (values_are_keys ? 1 : 2) * num_kv_heads;
     if (head_dim <= 0 || head_dim > kPrepareMaxHead || rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2 != 0 ||
         row_width < heads * head_dim || num_heads < 0 || num_kv_heads < 0 || page_size <= 0 || bias_width < 0 ||
@@ -228,7 +262,7 @@ WLLM_API int wllm_head_prepare(void* rows, int is_bf16, int row_width, const flo
     head_prepare_kernel<T, FOUR><<<grid, kWave * kPrepareWaves, 0, stream>>>(                                       \
         static_cast<T*>(rows), row_width, parts, splits, static_cast<size_t>(split_stride), bias, bias_width, positions, \
         inv_freq, slots, static_cast<T*>(cache), num_pages, num_heads, num_kv_heads, head_dim, rotary_dim, interleaved, \
-        norm_eps, norm_dim, values_are_keys, page_size, head_pieces)
+        norm_eps, norm_dim, values_are_keys, page_size, head_pieces, pre_q, pre_k, pre_eps, rot_scale)
     if (is_bf16) {
         if (four) LAUNCH(bf16, true); else LAUNCH(bf16, false);
     } else {

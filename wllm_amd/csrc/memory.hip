@@ -61,6 +61,45 @@ WLLM_API int wllm_memory_inputs(const void* row, long long row_stride, const int
     return launch_status();
 }
 
+// ---- a forget gate a channel that also decides what is written (the gating of HGRN2): from a row that begins
+// with the query heads and then the forget gate's projection z (heads * D columns each),
+//   f = lower + (1 - lower) * sigmoid(z + bias),   qkf[0] = act(q) (0: as it is, 1: silu),   qkf[1] = 1 - f,   qkf[2] = f
+// all float32: the recurrence S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T then is `memory_scan` with 1 - f in the
+// keys' place and f as a decay a row. ----
+template <typename T>
+__global__ void __launch_bounds__(256)
+memory_forget_inputs_kernel(const T* __restrict__ row, long long row_stride, const float* __restrict__ bias,
+                            const float* __restrict__ lower, float* __restrict__ qkf, int tokens, int width, int q_act) {
+    const int token = blockIdx.x;
+    const T* r = row + static_cast<size_t>(token) * row_stride;
+    const size_t plane = static_cast<size_t>(tokens) * width;
+    for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < width; e += gridDim.y * blockDim.x) {
+        const float q = to_float(r[e]);
+        const float z = to_float(r[width + e]) + (bias ? bias[e] : 0.f);
+        const float l = lower ? lower[e] : 0.f;
+        const float f = l + (1.f - l) * (1.f / (1.f + expf(-z)));
+        const size_t at = static_cast<size_t>(token) * width + e;
+        qkf[at] = q_act == 1 ? q / (1.f + expf(-q)) : q;
+        qkf[plane + at] = 1.f - f;
+        qkf[2 * plane + at] = f;
+    }
+}
+
+WLLM_API int wllm_memory_forget_inputs(const void* row, long long row_stride, const float* bias, const float* lower,
+                                       float* qkf, int is_bf16, int tokens, int width, int q_act, hipStream_t stream) {
+    if (tokens <= 0) return 0;
+    if (width <= 0 || q_act < 0 || q_act > 1) return -1;
+    const int tiles = (width + 255) / 256 < 64 ? (width + 255) / 256 : 64;
+    const dim3 grid(tokens, tiles);
+    if (is_bf16)
+        memory_forget_inputs_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(row), row_stride, bias, lower,
+                                                                    qkf, tokens, width, q_act);
+    else
+        memory_forget_inputs_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(row), row_stride, bias, lower,
+                                                                     qkf, tokens, width, q_act);
+    return launch_status();
+}
+
 // ---- exponential gates held in range by a running maximum.  Per head and token, with the gate
 // projections z_i, z_f (a band [n, 2 * heads] of a wider row: the input gates, then the forget gates):
 //   i = cap * tanh((z_i + bias_i) / cap)                 (cap <= 0: no cap)
@@ -155,7 +194,7 @@ constexpr int kMemCols = 16;
 constexpr int kMemSlices = kMemWaves * (kWave / kMemCols);
 constexpr int kMemThreads = kWave * kMemWaves;
 
-template <typename T, int R>
+template <typename T, int R, bool ROWS>
 __global__ void __launch_bounds__(kMemThreads)
 memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long long v_stride, const float* __restrict__ steps,
                    const float* __restrict__ decays, float* __restrict__ state, long long state_stride, long long n_offset,
@@ -166,6 +205,7 @@ memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long l
     constexpr int kRowsPass = kMemThreads / kRow;          // tokens a pass covers
     __shared__ __align__(16) float q_s[kMemTokens * kRow];
     __shared__ __align__(16) float k_s[kMemTokens * kRow];
+    __shared__ __align__(16) float f_s[ROWS ? kMemTokens * kRow : 1];      // ROWS: a decay a row of S and token
     __shared__ float v_s[kMemTokens * kMemCols];
     __shared__ float a_s[kMemTokens], b_s[kMemTokens];
     __shared__ float part_s[kMemTokens * kMemWaves * kMemCols];
@@ -193,17 +233,19 @@ memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long l
     // k (zeros beyond d: a row of S that is not there stays zero and adds nothing), one value of v, one token's a and b
     const int sj = tid % kRow, st = tid / kRow;
     const int vt = tid / kMemCols, vc = tid % kMemCols;
-    float q_r[kPasses], k_r[kPasses], v_r = 0.f, a_r = 1.f, b_r = 1.f;
+    float q_r[kPasses], k_r[kPasses], f_r[ROWS ? kPasses : 1], v_r = 0.f, a_r = 1.f, b_r = 1.f;
     auto fetch = [&](int t0) {
         const int count = min(kMemTokens, q_len - t0);
 #pragma unroll
         for (int u = 0; u < kPasses; ++u) {
             const int t = st + u * kRowsPass;
             q_r[u] = k_r[u] = 0.f;
+            if (ROWS) f_r[u] = 0.f;
             if (sj < d && t < count) {
                 const size_t at = static_cast<size_t>(q_start + t0 + t) * width + static_cast<size_t>(h) * d + sj;
                 q_r[u] = qk[at];
                 k_r[u] = qk[static_cast<size_t>(tokens) * width + at];
+                if (ROWS) f_r[u] = qk[2 * static_cast<size_t>(tokens) * width + at];
             }
         }
         if (tid < kMemTokens * kMemCols) {
@@ -226,6 +268,7 @@ memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long l
         for (int u = 0; u < kPasses; ++u) {
             q_s[(st + u * kRowsPass) * kRow + sj] = q_r[u];
             k_s[(st + u * kRowsPass) * kRow + sj] = k_r[u];
+            if (ROWS) f_s[(st + u * kRowsPass) * kRow + sj] = f_r[u];
         }
         if (tid < kMemTokens * kMemCols) v_s[tid] = v_r;
         if (tid < kMemTokens) {
@@ -237,10 +280,11 @@ memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long l
         const float a = a_s[t], bv = b_s[t] * v_s[t * kMemCols + col];
         const float* kt = k_s + t * kRow + n0;
         const float* qt = q_s + t * kRow + n0;
+        const float* ft = f_s + (ROWS ? t * kRow + n0 : 0);
         float part = 0.f;
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-            s[i] = fmaf(a, s[i], bv * kt[i]);
+            s[i] = fmaf(ROWS ? ft[i] : a, s[i], bv * kt[i]);
             part = fmaf(s[i], qt[i], part);
         }
         part = sum_across(sum_across(part, 32), 16);      // the wavefront's four slices of this column
@@ -280,28 +324,33 @@ memory_scan_kernel(const float* __restrict__ qk, const T* __restrict__ v, long l
 }
 
 // `steps` (float32 [3, tokens, heads], of which a and b are read; then `nq` float32 [tokens, heads] takes the
-// normaliser's sums and the normaliser lies at `n_offset` of a request's row) or, if null, `decays` (float32 [heads]; b = 1).
+// normaliser's sums and the normaliser lies at `n_offset` of a request's row) or, if null, `decays` (float32 [heads]; b = 1),
+// or, with `row_decays`, neither: then qk has a third plane [tokens, heads * d] of decays a row and token (b = 1).
 WLLM_API int wllm_memory_scan(const float* qk, const void* v, long long v_stride, const float* steps, const float* decays,
                               float* state, long long state_stride, long long n_offset, const int* seg_q_start,
                               const int* seg_q_len, const int* state_slots, float* y, float* nq, int is_bf16, int tokens,
-                              int segments, int heads, int d, int p_dim, hipStream_t stream) {
+                              int segments, int heads, int d, int p_dim, int row_decays, hipStream_t stream) {
     if (segments <= 0 || tokens <= 0) return 0;
-    if ((!steps) == (!decays) || (steps && !nq)) return -1;
+    if (row_decays ? (steps || decays) : ((!steps) == (!decays) || (steps && !nq))) return -1;
     if (heads <= 0 || d <= 0 || d > 8 * kMemSlices || p_dim <= 0) return -1;
     if (segments > 65535 || (p_dim + kMemCols) / kMemCols > 65535) return -1;
     const int r = (d + kMemSlices - 1) / kMemSlices;
     const int columns = p_dim + (steps ? 1 : 0);
     const dim3 grid(heads, segments, (columns + kMemCols - 1) / kMemCols);
-#define LAUNCH(T, R)                                                                                                \
-    memory_scan_kernel<T, R><<<grid, kMemThreads, 0, stream>>>(qk, static_cast<const T*>(v), v_stride, steps, decays, \
-                                                               state, state_stride, n_offset, seg_q_start, seg_q_len, \
-                                                               state_slots, y, nq, tokens, heads, d, p_dim)
-#define LAUNCH_R(T)                        \
-    if (r <= 1) LAUNCH(T, 1);              \
-    else if (r <= 2) LAUNCH(T, 2);         \
-    else if (r <= 4) LAUNCH(T, 4);         \
-    else LAUNCH(T, 8);
-    if (is_bf16) { LAUNCH_R(bf16) } else { LAUNCH_R(float) }
+#define LAUNCH(T, R, ROWS)                                                                                          \
+    memory_scan_kernel<T, R, ROWS><<<grid, kMemThreads, 0, stream>>>(qk, static_cast<const T*>(v), v_stride, steps, decays, \
+                                                                     state, state_stride, n_offset, seg_q_start, seg_q_len, \
+                                                                     state_slots, y, nq, tokens, heads, d, p_dim)
+#define LAUNCH_R(T, ROWS)                  \
+    if (r <= 1) LAUNCH(T, 1, ROWS);        \
+    else if (r <= 2) LAUNCH(T, 2, ROWS);   \
+    else if (r <= 4) LAUNCH(T, 4, ROWS);   \
+    else LAUNCH(T, 8, ROWS);
+    if (row_decays) {
+        if (is_bf16) { LAUNCH_R(bf16, true) } else { LAUNCH_R(float, true) }
+    } else {
+        if (is_bf16) { LAUNCH_R(bf16, false) } else { LAUNCH_R(float, false) }
+    }
 #undef LAUNCH_R
 #undef LAUNCH
     return launch_status();
@@ -310,7 +359,7 @@ WLLM_API int wllm_memory_scan(const float* qk, const void* v, long long v_stride
 // ---- out = o / rms_of_the_head(o) * weight * act(gate) * scale with o = y / den: the recurrence's sums (float32),
 // divided by the head's denominator den = max(|nq|, floor) + den_eps if there is one (nq, floor float32 [tokens, heads]),
 // every head divided by its own root mean square (eps inside the root), times a weight over the whole row (if
-// any), times the gate's activation (0: sigmoid, 1: silu) of a band of a wider row; out (the activation
+// any), times the gate's activation (0: sigmoid, 1: silu; 2: there is no gate) of a band of a wider row; out (the activation
 // type) may be a band too.  One wavefront a (token, head). ----
 template <typename T, int GATE>
 __global__ void __launch_bounds__(kWave)
@@ -328,14 +377,17 @@ head_norm_gate_kernel(const float* __restrict__ y, const T* __restrict__ gate, l
         ss = fmaf(o, o, ss);
     }
     const float inv = 1.f / sqrtf(wave_sum(ss) / static_cast<float>(p_dim) + eps);
-    const T* g = gate + static_cast<size_t>(token) * gate_stride + static_cast<size_t>(h) * p_dim;
+    const T* g = GATE == 2 ? nullptr : gate + static_cast<size_t>(token) * gate_stride + static_cast<size_t>(h) * p_dim;
     T* o = out + static_cast<size_t>(token) * out_stride + static_cast<size_t>(h) * p_dim;
     for (int i = threadIdx.x; i < p_dim; i += kWave) {
-        const float z = to_float(g[i]);
-        const float sg = 1.f / (1.f + expf(-z));
         float val = yr[i] / den * inv;
         if (weight) val *= weight[h * p_dim + i];
-        o[i] = from_float<T>(val * (GATE == 0 ? sg : z * sg) * scale);
+        if (GATE != 2) {
+            const float z = to_float(g[i]);
+            const float sg = 1.f / (1.f + expf(-z));
+            val *= GATE == 0 ? sg : z * sg;
+        }
+        o[i] = from_float<T>(val * scale);
     }
 }
 
@@ -343,14 +395,15 @@ WLLM_API int wllm_head_norm_gate(const float* y, const void* gate, long long gat
                                  long long out_stride, const float* nq, const float* floor, float den_eps, int is_bf16,
                                  int gate_kind, int tokens, int heads, int p_dim, float eps, float scale, hipStream_t stream) {
     if (tokens <= 0) return 0;
-    if (heads <= 0 || heads > 65535 || p_dim <= 0 || gate_kind < 0 || gate_kind > 1 || (!nq) != (!floor)) return -1;
+    if (heads <= 0 || heads > 65535 || p_dim <= 0 || gate_kind < 0 || gate_kind > 2 || (!nq) != (!floor)) return -1;
+    if (gate_kind != 2 && !gate) return -1;
     const dim3 grid(tokens, heads);
 #define LAUNCH(T, G)                                                                                                   \
     head_norm_gate_kernel<T, G><<<grid, kWave, 0, stream>>>(y, static_cast<const T*>(gate), gate_stride, weight,       \
                                                             static_cast<T*>(out), out_stride, nq, floor, den_eps, heads, \
                                                             p_dim, eps, scale)
-    if (is_bf16) { if (gate_kind == 0) LAUNCH(bf16, 0); else LAUNCH(bf16, 1); }
-    else { if (gate_kind == 0) LAUNCH(float, 0); else LAUNCH(float, 1); }
+    if (is_bf16) { if (gate_kind == 0) LAUNCH(bf16, 0); else if (gate_kind == 1) LAUNCH(bf16, 1); else LAUNCH(bf16, 2); }
+    else { if (gate_kind == 0) LAUNCH(float, 0); else if (gate_kind == 1) LAUNCH(float, 1); else LAUNCH(float, 2); }
 #undef LAUNCH
     return launch_status();
 }

@@ -1,14 +1,15 @@
 // A mixture of gated feed-forward experts on a flat batch of tokens: the router, the plan that sorts a
 // step's (token, chosen expert) pairs by expert, and the two grouped products on the matrix cores.
 //
-//   router   z = W_r x (float32), s = softmax(z) over all experts; only experts of the `keep` best of
+//   router   z = W_r x (float32), s = softmax(z) over all experts (or, `scoring` 1, s = sigmoid(z) of each); only experts of the `keep` best of
 //            `groups` equal groups of neighbours (a group's score: its largest s) may be chosen; the `top`
-//            allowed experts with the largest s are chosen, weights s / (sum of the chosen + eps)
+//            allowed experts with the largest s are chosen, weights s / (sum of the chosen + eps) (or, `normalize` 0, s itself)
 //   plan     an assignment is a = token * top + slot.  The assignments of one expert lie together, in
 //            tiles of R rows (16, 32, 64 or 128; the last tile of an expert padded with -1):
 //            plan[0] = tiles in use; plan[1 + t] = expert of tile t; plan[1 + max_tiles + R t + r] = a or -1
-//   up       act[a] = activation(x[token] Wg_e^T) * (x[token] Wu_e^T)
-//   down     out[slot][token] = weight[a] * (act[a] Wd_e^T), float32: a stack of `top` partial sums that
+//   up       act[a] = activation(x[token] Wg_e^T) * (x[token] Wu_e^T); with `in_weights` both products are multiplied by
+//            in_weights[a] first: the expert's input is in_weights[a] * x[token] (the factor taken out of the sums)
+//   down     out[slot][token] = weight[a] * (act[a] Wd_e^T) (weight 1 without `weights`), float32: a stack of `top` partial sums that
 //            whoever adds the feed-forward to the stream adds in order
 // A row's sums run over k in ascending chunks whatever tile the row lies in, so a token's result does
 // not depend on what else the batch holds.  Nothing is read on the host: the grid has room for the most
@@ -34,7 +35,7 @@ __device__ __forceinline__ int wave_lowest(int v) { return -static_cast<int>(wav
 template <typename T>
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const T* __restrict__ x, const float* __restrict__ router, int* __restrict__ ids, float* __restrict__ weights,
-                 int tokens, int width, int experts, int top, int groups, int keep, float eps) {
+                 int tokens, int width, int experts, int top, int groups, int keep, float eps, int scoring, int normalize) {
     __shared__ float z_s[kMoeMaxExperts];
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int token = blockIdx.x;
@@ -70,12 +71,27 @@ moe_route_kernel(const T* __restrict__ x, const float* __restrict__ router, int*
     }
     mx = wave_max(mx);
     float sum = 0.f;
+    if (scoring == 1) {
+        // a score of each expert by itself: in the terms of the softmax's code below, exp(z - mx) / sum with mx = 0
+        // and sum = 1 would not do (it overflows), so the sigmoid is written into sc and z_s as it is
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int j = 0; j < kRoutePer; ++j) {
-        sc[j] = lane + kWave * j < experts ? expf(sc[j] - mx) : 0.f;
-        sum += sc[j];
+        for (int j = 0; j < kRoutePer; ++j) {
+            const int e = lane + kWave * j;
+            sc[j] = e < experts ? 1.f / (1.f + expf(-sc[j])) : 0.f;
+            if (e < experts) z_s[e] = sc[j];
+        }
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        sum = 1.f;
+    } else {
+#pragma unroll
+        for (int j = 0; j < kRoutePer; ++j) {
+            sc[j] = lane + kWave * j < experts ? expf(sc[j] - mx) : 0.f;
+            sum += sc[j];
+        }
+        sum = wave_sum(sum);
     }
-    sum = wave_sum(sum);
     // a score that may still be chosen is >= 0; one that may not is -1
 #pragma unroll
     for (int j = 0; j < kRoutePer; ++j) sc[j] = lane + kWave * j < experts ? sc[j] / sum : -1.f;
@@ -89,7 +105,8 @@ moe_route_kernel(const T* __restrict__ x, const float* __restrict__ router, int*
             gs[j] = -1.f;
             allowed[j] = false;
             if (g < groups)
-                for (int m = 0; m < per; ++m) gs[j] = fmaxf(gs[j], expf(z_s[g * per + m] - mx) / sum);
+                for (int m = 0; m < per; ++m)
+                    gs[j] = fmaxf(gs[j], scoring == 1 ? z_s[g * per + m] : expf(z_s[g * per + m] - mx) / sum);
         }
         for (int pick = 0; pick < keep; ++pick) {
             float best = -1.f;
@@ -133,24 +150,26 @@ moe_route_kernel(const T* __restrict__ x, const float* __restrict__ router, int*
             wt[slot] = best;
         }
     }
-    if (lane == 0) {
+    if (lane == 0 && normalize) {
         const float denom = chosen_sum + eps;
         for (int slot = 0; slot < top; ++slot) wt[slot] /= denom;
     }
 }
 
 WLLM_API int wllm_moe_route(const void* x, const float* router, int* ids, float* weights, int is_bf16, int tokens, int width,
-                            int experts, int top, int groups, int keep, float eps, hipStream_t stream) {
+                            int experts, int top, int groups, int keep, float eps, int scoring, int normalize,
+                            hipStream_t stream) {
     if (tokens <= 0) return 0;
+    if (scoring < 0 || scoring > 1) return -1;
     if (experts <= 0 || experts > kMoeMaxExperts || groups <= 0 || experts % groups || keep <= 0 || keep > groups || top <= 0 ||
         top > keep * (experts / groups) || width <= 0)
         return -1;
     if (is_bf16)
         moe_route_kernel<bf16><<<tokens, 256, 0, stream>>>(static_cast<const bf16*>(x), router, ids, weights, tokens, width,
-                                                           experts, top, groups, keep, eps);
+                                                           experts, top, groups, keep, eps, scoring, normalize);
     else
         moe_route_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<const float*>(x), router, ids, weights, tokens, width,
-                                                            experts, top, groups, keep, eps);
+                                                            experts, top, groups, keep, eps, scoring, normalize);
     return launch_status();
 }
 
@@ -268,7 +287,7 @@ template <> struct MoeFrag<float> {
 template <typename T, int ACT, int MT>
 __global__ void __launch_bounds__(256)
 moe_up_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ tiles, const int* __restrict__ plan,
-              int max_tiles, T* __restrict__ act, int K, int ff, int top) {
+              int max_tiles, T* __restrict__ act, int K, int ff, int top, const float* __restrict__ in_weights) {
     constexpr int U = MT == 4 ? 2 : 4;          // chunks whose loads are asked for before the first product
     const int tile = blockIdx.x;
     if (tile >= plan[0]) return;
@@ -342,17 +361,19 @@ moe_up_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __restr
     for (int m = 0; m < MT; ++m) {
         if (a_i[m] < 0) continue;
         T* out = act + static_cast<size_t>(a_i[m]) * ff;
+        const float scale = in_weights ? in_weights[a_i[m]] : 1.f;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int c = c0 + 4 * g + v;
-            if (c < ff) out[c] = from_float<T>(activate<ACT>(acc_g[m][v]) * acc_u[m][v]);
+            if (c < ff) out[c] = from_float<T>(activate<ACT>(acc_g[m][v] * scale) * (acc_u[m][v] * scale));
         }
     }
 }
 
 // `tile_rows`: the rows of the plan's tiles, 16, 32 or 64.
 WLLM_API int wllm_moe_up(const void* x, const void* w, const void* tiles, const int* plan, int max_tiles, int tile_rows,
-                         void* act, int is_bf16, int activation, int K, int ff, int top, hipStream_t stream) {
+                         void* act, int is_bf16, int activation, int K, int ff, int top, const float* in_weights,
+                         hipStream_t stream) {
     if (max_tiles <= 0) return 0;
     if (K <= 0 || ff <= 0 || top <= 0 || activation < 0 || activation >= kActivations || (ff + 63) / 64 > 65535) return -1;
     if (tile_rows != 16 && tile_rows != 32 && tile_rows != 64) return -1;
@@ -361,7 +382,7 @@ WLLM_API int wllm_moe_up(const void* x, const void* w, const void* tiles, const 
 #define LAUNCH_MT(T, MT)                                                                                              \
     WLLM_BY_ACTIVATION(activation, (moe_up_kernel<T, ACT, MT><<<grid, 256, 0, stream>>>(                              \
                                        static_cast<const T*>(x), static_cast<const T*>(w), static_cast<const T*>(tiles), \
-                                       plan, max_tiles, static_cast<T*>(act), K, ff, top)))
+                                       plan, max_tiles, static_cast<T*>(act), K, ff, top, in_weights)))
 #define LAUNCH(T)                                    \
     if (tile_rows == 16) { LAUNCH_MT(T, 1); }        \
     else if (tile_rows == 32) { LAUNCH_MT(T, 2); }   \
@@ -438,7 +459,7 @@ moe_down_kernel(const T* __restrict__ act, const T* __restrict__ w, const T* __r
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         if (a_i[m] < 0) continue;
-        const float weight = weights[a_i[m]];
+        const float weight = weights ? weights[a_i[m]] : 1.f;
         float* o = out + (static_cast<size_t>(a_i[m] % top) * tokens + a_i[m] / top) * width;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
@@ -504,6 +525,8 @@ __global__ void __launch_bounds__(256, 2)
 moe_tile_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const int* __restrict__ plan, int max_tiles,
                 bf16* __restrict__ act, float* __restrict__ out32, const float* __restrict__ weights, int N, int K, int top,
                 int tokens) {
+    // (`weights`: of the second product the factor of a row's result, 1 if null; of the first the factor of a row's
+    // input, taken out of both sums, none if null)
     constexpr int kWaves = 4, kStages = 2;
     constexpr int kWBytes = kBigRows * kBigRowBytes;
     constexpr int kLoads = 2 * kBigRows / 8 / kWaves;
@@ -593,16 +616,18 @@ moe_tile_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const in
         if (asg < 0) continue;
         if (GATED) {
             bf16* o_row = act + static_cast<size_t>(asg) * N;
+            const float scale = weights ? weights[asg] : 1.f;
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
                 const int n = n_base + wn * 32 + 16 * a + 4 * g;
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
                     if (n + v < N)
-                        o_row[n + v] = from_float<bf16>(activate<(GATED > 0 ? GATED - 1 : 0)>(acc[a][b][v]) * acc[a + 2][b][v]);
+                        o_row[n + v] = from_float<bf16>(activate<(GATED > 0 ? GATED - 1 : 0)>(acc[a][b][v] * scale) *
+                                                        (acc[a + 2][b][v] * scale));
             }
         } else {
-            const float weight = weights[asg];
+            const float weight = weights ? weights[asg] : 1.f;
             float* o_row = out32 + (static_cast<size_t>(asg % top) * tokens + asg / top) * N;
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
@@ -624,7 +649,7 @@ WLLM_API int wllm_moe_tiles(const void* x, const void* w, const int* plan, int m
     if (max_tiles <= 0 || x_rows <= 0) return 0;
     if (N <= 0 || K < kBigKeys || K % kBigKeys || top <= 0 || tokens <= 0 || activation >= kActivations) return -1;
     const bool gated = activation >= 0;
-    if ((gated && !act) || (!gated && (!out32 || !weights))) return -1;
+    if ((gated && !act) || (!gated && !out32)) return -1;
     if (static_cast<size_t>(gated ? 2 : 1) * N * K * 2 >= (size_t(1) << 32) || static_cast<size_t>(x_rows) * K * 2 >= (size_t(1) << 32))
         return -1;
     const int columns = gated ? kBigRows / 2 : kBigRows;

@@ -83,6 +83,53 @@ WLLM_API int wllm_causal_conv(const void* in, long long in_stride, const float* 
     return launch_status();
 }
 
+// ---- the same convolution on the residual stream itself, in front of a sublayer that reads the stream:
+// out[t, c] = x[t, c] + sum_k w[c, k] * x[t - (taps - 1) + k, c], float32 sums in this order, no bias and no
+// activation; x float32 [tokens, channels], out the activation type.  The carried rows (the request's last
+// taps - 1 rows of x, the oldest first) are kept by `conv_carry_kernel`, as above. ----
+template <typename T>
+__global__ void __launch_bounds__(256)
+stream_conv_kernel(const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ state,
+                   long long state_stride, long long carried_offset, const int* __restrict__ token_segment,
+                   const int* __restrict__ seg_q_start, const int* __restrict__ state_slots, T* __restrict__ out,
+                   int channels, int taps) {
+    const int token = blockIdx.x;
+    const int seg = token_segment[token];
+    const int local = token - seg_q_start[seg];
+    const float* carried = state + static_cast<size_t>(state_slots[seg]) * state_stride + carried_offset;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
+        float acc = x[static_cast<size_t>(token) * channels + c];
+        for (int k = 0; k < taps; ++k) {
+            const int src = local - (taps - 1) + k;
+            const float v = src >= 0 ? x[static_cast<size_t>(token - local + src) * channels + c]
+                                     : carried[static_cast<size_t>(taps - 1 + src) * channels + c];
+            acc = fmaf(weight[static_cast<size_t>(c) * taps + k], v, acc);
+        }
+        out[static_cast<size_t>(token) * channels + c] = from_float<T>(acc);
+    }
+}
+
+WLLM_API int wllm_stream_conv(const float* x, const float* weight, float* state, long long state_stride,
+                              long long carried_offset, const int* token_segment, const int* seg_q_start,
+                              const int* seg_q_len, const int* state_slots, void* out, int out_bf16, int tokens,
+                              int segments, int channels, int taps, hipStream_t stream) {
+    if (tokens <= 0 || segments <= 0) return 0;
+    if (channels <= 0 || taps < 1 || taps > 64) return -1;
+    const int tiles = (channels + 255) / 256 < 64 ? (channels + 255) / 256 : 64;
+    const dim3 grid(tokens, tiles), carry_grid(segments, tiles);
+    if (out_bf16)
+        stream_conv_kernel<bf16><<<grid, 256, 0, stream>>>(x, weight, state, state_stride, carried_offset, token_segment,
+                                                           seg_q_start, state_slots, static_cast<bf16*>(out), channels, taps);
+    else
+        stream_conv_kernel<float><<<grid, 256, 0, stream>>>(x, weight, state, state_stride, carried_offset, token_segment,
+                                                            seg_q_start, state_slots, static_cast<float*>(out), channels, taps);
+    if (const int err = launch_status()) return err;
+    if (taps == 1) return 0;
+    conv_carry_kernel<float><<<carry_grid, 256, 0, stream>>>(x, channels, state, state_stride, carried_offset, seg_q_start,
+                                                             seg_q_len, state_slots, channels, taps);
+    return launch_status();
+}
+
 // ---- the recurrence.  Per head h (group g = h / (heads / groups)), token by token:
 //   dt = softplus(dt_in + dt_bias[h]);  S = exp(-exp(A_log[h]) * dt) * S + dt * B_t x_t^T;  y_t = S^T C_t + D[h] x_t
 // with S [N, P], B_t and C_t [N] of the group, x_t [P] of the head.  xbc [tokens, heads*P + 2*groups*N]

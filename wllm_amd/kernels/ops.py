@@ -361,7 +361,8 @@ def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: to
                  inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor], cache: Optional[torch.Tensor], *,
                  num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, interleaved: bool = False,
                  norm_eps: Optional[float] = None, values_are_keys: bool = False,
-                 parts: Optional[torch.Tensor] = None, norm_dim: Optional[int] = None) -> None:
+                 parts: Optional[torch.Tensor] = None, norm_dim: Optional[int] = None,
+                 head_norm: Optional[tuple] = None, rot_scale: float = 1.0) -> None:
     """What `rope_and_cache_write` does, for attention blocks that do more between projection and
     attention.  rows T [n, width]: num_heads query heads, num_kv_heads key heads, num_kv_heads value
     heads unless `values_are_keys`, then any further columns.  In this order, in float32: every
@@ -373,7 +374,10 @@ def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: to
     `interleaved`, else (j, j + len(inv_freq)); with `norm_eps` every query and key head is
     divided by sqrt(sum of its squares / norm_dim + norm_eps) (norm_dim: head_dim unless given; less where
     the last elements of every head are padding that is always zero); the heads are written back and the
-    key heads stored.  slots, cache as in `rope_and_cache_write` (both None: nothing is stored)."""
+    key heads stored.  slots, cache as in `rope_and_cache_write` (both None: nothing is stored).
+    `head_norm` = (w_q, w_k, eps), float32 [head_dim] each: before the rotation every query head is divided by
+    sqrt(sum of its squares / norm_dim + eps) and multiplied by w_q, every key head likewise by w_k (an RMS
+    norm with a weight over each head).  `rot_scale`: sine and cosine are multiplied by it."""
     heads = num_heads + (1 if values_are_keys else 2) * num_kv_heads
     _dense(rows, "rows", _ACT)
     _need(rows.dim() == 2 and rows.shape[1] >= heads * head_dim,
@@ -400,9 +404,18 @@ def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: to
         _dense(cache, "cache", rows.dtype)
         _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (2, num_kv_heads, page_size * head_dim),
               lambda: f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
+    extra = {}
+    if head_norm is not None:
+        w_q, w_k, pre_eps = head_norm
+        _dense(w_q, "head_norm[0]", torch.float32, (head_dim,))
+        _dense(w_k, "head_norm[1]", torch.float32, (head_dim,))
+        _need(pre_eps >= 0.0, "head_norm: eps must not be negative")
+        extra["head_norm"] = (w_q, w_k, float(pre_eps))
+    if rot_scale != 1.0:
+        extra["rot_scale"] = float(rot_scale)
     if n:
         call("head_prepare", rows, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim,
-             page_size, bool(interleaved), norm_eps, bool(values_are_keys), parts, norm_dim)
+             page_size, bool(interleaved), norm_eps, bool(values_are_keys), parts, norm_dim, **extra)
 
 
 def _band(t: torch.Tensor, name: str, dtype, rows: int, cols: int) -> None:
@@ -832,6 +845,29 @@ def causal_conv(inp: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, sta
              state_slots, out)
 
 
+def stream_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, carried_offset: int, token_segment: torch.Tensor,
+                seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor) -> None:
+    """A short causal convolution over time on each channel of the residual stream, added to the stream's own value:
+    out[t, c] = x[t, c] + sum_k weight[c, k] * x[t - (taps - 1) + k, c], the rows before a segment's first token taken
+    from the request's carried rows (zeros for a fresh request), which afterwards hold the segment's last taps - 1 rows.
+    x float32 [n, C]; weight float32 [C, taps]; state float32 [slots, W] with the carried rows [taps - 1, C] from column
+    `carried_offset` of row state_slots[segment]; out T [n, C].  float32 sums in the order written."""
+    _dense(x, "x", torch.float32)
+    _need(x.dim() == 2, "x: expected [n, channels]")
+    n, channels = x.shape
+    _dense(weight, "weight", torch.float32)
+    _need(weight.dim() == 2 and weight.shape[0] == channels and 1 <= weight.shape[1] <= 64, "weight: expected [channels, taps <= 64]")
+    taps = weight.shape[1]
+    _dense(state, "state", torch.float32)
+    _need(state.dim() == 2 and 0 <= carried_offset and carried_offset + (taps - 1) * channels <= state.shape[1],
+          "state: a row holds the carried rows from carried_offset")
+    _dense(token_segment, "token_segment", torch.int32, (n,))
+    _segments(seg_q_start, seg_q_len, state_slots)
+    _dense(out, "out", _ACT, (n, channels))
+    if n:
+        call("stream_conv", x, weight, state, int(carried_offset), token_segment, seg_q_start, seg_q_len, state_slots, out)
+
+
 def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
              state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor,
              y: torch.Tensor, *, heads: int, groups: int, state_size: int, head_dim: int,
@@ -887,7 +923,8 @@ def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, out
 
 
 # ---- a matrix memory a head (linear attention in its recurrent form) ------------------------------------
-GATE_KINDS = {"sigmoid": 0, "silu": 1}
+GATE_KINDS = {"sigmoid": 0, "silu": 1, "none": 2}
+QUERY_ACTIVATIONS = {"none": 0, "silu": 1}
 
 
 def _segments(seg_q_start, seg_q_len, state_slots) -> int:
@@ -918,6 +955,24 @@ def memory_inputs(row: torch.Tensor, positions: torch.Tensor, inv_freq: Optional
         call("memory_inputs", row, positions, inv_freq, qk, heads, head_dim, float(q_scale), float(k_scale))
 
 
+def memory_forget_inputs(row: torch.Tensor, bias: Optional[torch.Tensor], lower: Optional[torch.Tensor], qkf: torch.Tensor, *,
+                         width: int, q_activation: str = "none") -> None:
+    """The inputs of a recurrence whose forget gate a channel also decides what is written.  row T [n, >= 2 * width]
+    (may be a band) begins with the queries and then the gate's projection z; bias, lower float32 [width] or None.
+    f = lower + (1 - lower) * sigmoid(z + bias);  qkf[0] = act(q) ("none" or "silu"), qkf[1] = 1 - f, qkf[2] = f, all
+    float32 [3, n, width]: what `memory_scan(row_decays=True)` takes."""
+    _need(q_activation in QUERY_ACTIVATIONS, lambda: f"q_activation {q_activation!r}: one of {sorted(QUERY_ACTIVATIONS)}")
+    _need(row.dim() == 2 and row.dtype in _ACT, "row: expected T [n, >= 2 * width]")
+    n = row.shape[0]
+    _band(row[:, :2 * width], "row", row.dtype, n, 2 * width)
+    for t, name in ((bias, "bias"), (lower, "lower")):
+        if t is not None:
+            _dense(t, name, torch.float32, (width,))
+    _dense(qkf, "qkf", torch.float32, (3, n, width))
+    if n:
+        call("memory_forget_inputs", row, bias, lower, qkf, width, q_activation)
+
+
 def memory_gates(gates: torch.Tensor, i_bias: Optional[torch.Tensor], f_bias: Optional[torch.Tensor], state: torch.Tensor,
                  m_offset: int, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor,
                  steps: torch.Tensor, *, heads: int, cap: Optional[float] = None) -> None:
@@ -945,20 +1000,25 @@ def memory_gates(gates: torch.Tensor, i_bias: Optional[torch.Tensor], f_bias: Op
 def memory_scan(qk: torch.Tensor, v: torch.Tensor, steps: Optional[torch.Tensor], decays: Optional[torch.Tensor],
                 state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor,
                 y: torch.Tensor, *, heads: int, head_dim: int, value_dim: int, nq: Optional[torch.Tensor] = None,
-                n_offset: int = 0) -> None:
+                n_offset: int = 0, row_decays: bool = False) -> None:
     """The matrix memory's recurrence over each segment's tokens in order, from and into the request's
     carried state.  Per head:  S = a S + b k v^T;  y = S^T q  with (a, b) of the token from `steps` (float32
     [3, n, heads], of which the first two are read) or, with `decays` (float32 [heads]) instead, (decays[h], 1).
     With `steps` the normaliser n = a n + b k is carried too, as [heads, head_dim] from column `n_offset` of the
     request's row, and nq (float32 [n, heads]) takes n . q.  qk float32 [2, n, heads * head_dim]: queries, then
     keys; v T [n, heads * value_dim] (may be a band); state float32 [slots, W], whose row state_slots[segment]
-    begins with S as [heads, head_dim, value_dim]; y float32 [n, heads * value_dim].  All of the recurrence is float32."""
-    _need((steps is None) != (decays is None), "steps or decays, one of the two")
+    begins with S as [heads, head_dim, value_dim]; y float32 [n, heads * value_dim].  All of the recurrence is float32.
+    `row_decays` (then neither `steps` nor `decays`): qk has a third plane, float32 [3, n, heads * head_dim], of decays a
+    row of S and token: S[i, :] = qk[2][i] S[i, :] + k[i] v^T."""
+    if row_decays:
+        _need(steps is None and decays is None, "row_decays: neither steps nor decays")
+    else:
+        _need((steps is None) != (decays is None), "steps or decays, one of the two")
     _need(v.dim() == 2 and v.dtype in _ACT, "v: expected T [n, heads * value_dim]")
     n = v.shape[0]
     _band(v, "v", v.dtype, n, heads * value_dim)
     _need(0 < head_dim <= 256 and value_dim > 0, "head_dim: from 1 to 256")
-    _dense(qk, "qk", torch.float32, (2, n, heads * head_dim))
+    _dense(qk, "qk", torch.float32, (3 if row_decays else 2, n, heads * head_dim))
     _dense(state, "state", torch.float32)
     memory = heads * head_dim * value_dim
     _need(state.dim() == 2 and state.shape[1] >= memory, "state: a row holds at least [heads, D, P]")
@@ -968,29 +1028,33 @@ def memory_scan(qk: torch.Tensor, v: torch.Tensor, steps: Optional[torch.Tensor]
         _dense(nq, "nq", torch.float32, (n, heads))
         _need(memory <= n_offset and n_offset + heads * head_dim <= state.shape[1], "state: the normaliser lies behind S")
     else:
-        _dense(decays, "decays", torch.float32, (heads,))
+        if not row_decays:
+            _dense(decays, "decays", torch.float32, (heads,))
         _need(nq is None, "nq: only with steps")
     _segments(seg_q_start, seg_q_len, state_slots)
     _dense(y, "y", torch.float32, (n, heads * value_dim))
     if n:
         call("memory_scan", qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads, head_dim, value_dim, nq,
-             int(n_offset))
+             int(n_offset), **({"row_decays": True} if row_decays else {}))
 
 
-def head_norm_gate(y: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], out: torch.Tensor, *, heads: int,
+def head_norm_gate(y: torch.Tensor, gate: Optional[torch.Tensor], weight: Optional[torch.Tensor], out: torch.Tensor, *, heads: int,
                    eps: float, activation: str = "sigmoid", scale: float = 1.0, nq: Optional[torch.Tensor] = None,
                    floor: Optional[torch.Tensor] = None, den_eps: float = 0.0) -> None:
     """out = o / rms_of_its_head(o) * weight * act(gate) * scale with o = y / den: every one of `heads` equal parts
     of a row of y is divided by its denominator den = max(|nq|, floor) + den_eps (nq, floor float32 [n, heads]; without
     them den = 1) and then by sqrt(mean of its squares + eps).  y float32 [n, W]; gate T [n, W] and out T [n, W]
-    may be bands of wider tensors; weight float32 [W] or None; activation "sigmoid" or "silu"."""
+    may be bands of wider tensors; weight float32 [W] or None; activation "sigmoid" or "silu", or "none" with gate None."""
     _need(activation in GATE_KINDS, lambda: f"activation {activation!r}: expected one of {sorted(GATE_KINDS)}")
     _dense(y, "y", torch.float32)
     _need(y.dim() == 2 and heads > 0 and y.shape[1] % heads == 0, "y: expected [n, heads * P]")
     n, w = y.shape
-    _need(gate.dtype in _ACT, "gate: expected T")
-    _band(gate, "gate", gate.dtype, n, w)
-    _band(out, "out", gate.dtype, n, w)
+    _need((gate is None) == (activation == "none"), "gate: None goes with the activation 'none'")
+    if gate is not None:
+        _need(gate.dtype in _ACT, "gate: expected T")
+        _band(gate, "gate", gate.dtype, n, w)
+    _need(out.dtype in _ACT and (gate is None or out.dtype == gate.dtype), "out: expected T")
+    _band(out, "out", out.dtype, n, w)
     if weight is not None:
         _dense(weight, "weight", torch.float32, (w,))
     _need((nq is None) == (floor is None), "nq and floor go together")
@@ -1032,13 +1096,18 @@ def moe_plan_size(assignments: int, experts: int, tile_rows: int = MOE_TILE_ROWS
     return 1 + moe_max_tiles(assignments, experts, tile_rows) * (1 + tile_rows)
 
 
+MOE_SCORINGS = {"softmax": 0, "sigmoid": 1}
+
+
 def moe_route(x: torch.Tensor, router: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, *, groups: int = 1,
-              keep: int = 1, eps: float = 1e-20) -> None:
+              keep: int = 1, eps: float = 1e-20, scoring: str = "softmax", normalize: bool = True) -> None:
     """Which experts each token uses.  z = x router^T in float32; s = softmax(z) over all experts; the
     experts form `groups` equal groups of neighbours, a group's score is its largest s, and only experts of
     the `keep` best groups may be chosen; the `top` = ids.shape[1] allowed experts with the largest s are
     chosen (of equal scores the lower index first), weights = their s / (sum of the chosen + eps).
+    `scoring` "sigmoid": s = sigmoid(z), every expert by itself.  `normalize` False: weights = the chosen s themselves.
     x T [n, width]; router float32 [experts, width]; ids int32 [n, top]; weights float32 [n, top]."""
+    _need(scoring in MOE_SCORINGS, lambda: f"scoring {scoring!r}: one of {sorted(MOE_SCORINGS)}")
     _dense(x, "x", _ACT)
     _need(x.dim() == 2, "x: expected [n, width]")
     n, width = x.shape
@@ -1053,7 +1122,8 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, ids: torch.Tensor, weights:
     _need(groups > 0 and experts % groups == 0 and 0 < keep <= groups, "groups must divide the experts; keep from 1 to groups")
     _need(0 < top <= keep * (experts // groups), "top: at most the experts of the kept groups")
     if n:
-        call("moe_route", x, router, ids, weights, int(groups), int(keep), float(eps))
+        extra = {} if scoring == "softmax" and normalize else {"scoring": scoring, "normalize": bool(normalize)}
+        call("moe_route", x, router, ids, weights, int(groups), int(keep), float(eps), **extra)
 
 
 def moe_plan(ids: torch.Tensor, plan: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS) -> None:
@@ -1087,11 +1157,14 @@ def _expert_tiles(tiles: Optional[torch.Tensor], w: torch.Tensor) -> None:
 
 
 def moe_experts_up(x: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, act: torch.Tensor, top: int,
-                   activation: str, tile_rows: int = MOE_TILE_ROWS, tiles: Optional[torch.Tensor] = None) -> None:
+                   activation: str, tile_rows: int = MOE_TILE_ROWS, tiles: Optional[torch.Tensor] = None,
+                   in_weights: Optional[torch.Tensor] = None) -> None:
     """act[a] = activation(x[a // top] Wg_e^T) * (x[a // top] Wu_e^T) for every assignment a of the plan (of tiles of
     `tile_rows` rows), e its expert.  x T [n, width]; w T [experts, 2 * ff, width]: an expert's gate rows, then its
     up rows; act T [n * top, ff]; float32 sums.  `tiles`: `tile_weight` of w as one matrix [experts * 2 * ff, width]
-    (ff a multiple of 16), which the kernel for tiles of 16 rows streams instead of w."""
+    (ff a multiple of 16), which the kernel for tiles of 16 rows streams instead of w.  `in_weights` (float32
+    [n, top]): the expert's input is in_weights.flat[a] * x[a // top]; the factor is taken out of both sums and
+    multiplied in, in float32, before the activation."""
     _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {sorted(ACTIVATIONS)}")
     _dense(x, "x", _ACT)
     _need(x.dim() == 2, "x: expected [n, width]")
@@ -1103,18 +1176,24 @@ def moe_experts_up(x: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, act: to
     _dense(plan, "plan", torch.int32, (moe_plan_size(n * top, experts, tile_rows),))
     _need(tiles is None or ff % 16 == 0, "tiles: ff must be a multiple of 16")
     _expert_tiles(tiles, w)
+    extra = {}
+    if in_weights is not None:
+        _dense(in_weights, "in_weights", torch.float32, (n, top))
+        extra["in_weights"] = in_weights
     if n:
         if _big_tiles(tile_rows, x.dtype, width):
-            call("moe_experts_up_tiled", x, w, plan, act, int(top), activation)
+            call("moe_experts_up_tiled", x, w, plan, act, int(top), activation, **extra)
         else:
-            call("moe_experts_up", x, w, plan, act, int(top), activation, tiles, int(tile_rows))
+            call("moe_experts_up", x, w, plan, act, int(top), activation, tiles, int(tile_rows), **extra)
 
 
 def moe_experts_down(act: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, weights: torch.Tensor,
-                     out: torch.Tensor, tile_rows: int = MOE_TILE_ROWS, tiles: Optional[torch.Tensor] = None) -> None:
+                     out: torch.Tensor, tile_rows: int = MOE_TILE_ROWS, tiles: Optional[torch.Tensor] = None,
+                     weighted: bool = True) -> None:
     """out[a % top][a // top] = weights.flat[a] * (act[a] Wd_e^T) for every assignment a of the plan: the
     experts' weighted results as a stack of `top` float32 partial sums over the tokens.  act T [n * top, ff];
-    w T [experts, width, ff]; weights float32 [n, top]; out float32 [top, n, width]."""
+    w T [experts, width, ff]; weights float32 [n, top]; out float32 [top, n, width] (or the first `top` slices of a
+    taller stack).  `weighted` False: the factor is 1 (the weights entered elsewhere)."""
     _dense(act, "act", _ACT)
     _need(act.dim() == 2, "act: expected [n * top, ff]")
     _dense(weights, "weights", torch.float32)
@@ -1125,11 +1204,12 @@ def moe_experts_down(act: torch.Tensor, w: torch.Tensor, plan: torch.Tensor, wei
     _dense(out, "out", torch.float32, (top, n, w.shape[1]))
     _dense(plan, "plan", torch.int32, (moe_plan_size(n * top, w.shape[0], tile_rows),))
     _expert_tiles(tiles, w)
+    extra = {} if weighted else {"weighted": False}
     if n:
         if _big_tiles(tile_rows, act.dtype, act.shape[1]):
-            call("moe_experts_down_tiled", act, w, plan, weights, out)
+            call("moe_experts_down_tiled", act, w, plan, weights, out, **extra)
         else:
-            call("moe_experts_down", act, w, plan, weights, out, tiles, int(tile_rows))
+            call("moe_experts_down", act, w, plan, weights, out, tiles, int(tile_rows), **extra)
 
 
 # ---- the framework's own operations that go through the same door as a part's ------------------
@@ -1153,17 +1233,20 @@ def _register_own() -> None:
 
 
     def prepare(fn, stream, rows, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim,
-                page_size, interleaved, norm_eps, values_are_keys, parts, norm_dim):
+                page_size, interleaved, norm_eps, values_are_keys, parts, norm_dim, head_norm=None, rot_scale=1.0):
+        w_q, w_k, pre_eps = head_norm if head_norm is not None else (None, None, -1.0)
         splits, stride = (parts.shape[0], parts.shape[1] * parts.shape[2]) if parts is not None else (0, 0)
         return fn(p(rows), int(rows.dtype == torch.bfloat16), rows.shape[1], p(parts), splits, stride, p(bias),
                   bias.shape[0] if bias is not None else 0, p(positions), p(inv_freq), p(slots), p(cache), cache.shape[0] if cache is not None else 0,
                   rows.shape[0], num_heads, num_kv_heads, head_dim,
                   2 * inv_freq.shape[0] if inv_freq is not None else 0, int(interleaved),
-                  float(norm_eps) if norm_eps is not None else -1.0, norm_dim, int(values_are_keys), page_size, stream)
+                  float(norm_eps) if norm_eps is not None else -1.0, norm_dim, int(values_are_keys), page_size,
+                  p(w_q), p(w_k), pre_eps, rot_scale, stream)
 
     register_op("head_prepare", entry_point="wllm_head_prepare",
                 argtypes=[c_void_p, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                          c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p],
+                          c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p,
+                          c_void_p, c_float, c_float, c_void_p],
                 launch=prepare)
     register_op("sigmoid_gate", entry_point="wllm_sigmoid_gate",
                 argtypes=[c_void_p, c_longlong, c_void_p, c_longlong, c_void_p, c_longlong, c_int, c_int, c_int, c_int,
@@ -1237,6 +1320,14 @@ def _register_own() -> None:
                     p(inp), inp.stride(0), p(weight), p(bias), p(state), state.stride(0), carried_offset, p(token_segment),
                     p(seg_q_start), p(seg_q_len), p(state_slots), p(out), int(inp.dtype == torch.bfloat16), inp.shape[0],
                     seg_q_start.shape[0], inp.shape[1], weight.shape[1], stream))
+    register_op("stream_conv", entry_point="wllm_stream_conv",
+                argtypes=[c_void_p, c_void_p, c_void_p, c_longlong, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_int, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, x, weight, state, carried_offset, token_segment, seg_q_start, seg_q_len, state_slots,
+                out: fn(
+                    p(x), p(weight), p(state), state.stride(0), carried_offset, p(token_segment), p(seg_q_start), p(seg_q_len),
+                    p(state_slots), p(out), int(out.dtype == torch.bfloat16), x.shape[0], seg_q_start.shape[0], x.shape[1],
+                    weight.shape[1], stream))
     register_op("ssm_scan", entry_point="wllm_ssm_scan",
                 argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p,
                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -1258,6 +1349,11 @@ def _register_own() -> None:
                 launch=lambda fn, stream, row, positions, inv_freq, qk, heads, head_dim, q_scale, k_scale: fn(
                     p(row), row.stride(0), p(positions), p(inv_freq), p(qk), bf(row), row.shape[0], heads, head_dim,
                     2 * inv_freq.shape[0] if inv_freq is not None else 0, q_scale, k_scale, stream))
+    register_op("memory_forget_inputs", entry_point="wllm_memory_forget_inputs",
+                argtypes=[c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, row, bias, lower, qkf, width, q_activation: fn(
+                    p(row), row.stride(0), p(bias), p(lower), p(qkf), bf(row), row.shape[0], width,
+                    QUERY_ACTIVATIONS[q_activation], stream))
     register_op("memory_gates", entry_point="wllm_memory_gates",
                 argtypes=[c_void_p, c_longlong, c_void_p, c_void_p, c_float, c_void_p, c_longlong, c_longlong, c_void_p,
                           c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
@@ -1268,49 +1364,50 @@ def _register_own() -> None:
                     seg_q_start.shape[0], heads, stream))
     register_op("memory_scan", entry_point="wllm_memory_scan",
                 argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_longlong, c_longlong, c_void_p,
-                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
                 launch=lambda fn, stream, qk, v, steps, decays, state, seg_q_start, seg_q_len, state_slots, y, heads,
-                head_dim, value_dim, nq=None, n_offset=0: fn(
+                head_dim, value_dim, nq=None, n_offset=0, row_decays=False: fn(
                     p(qk), p(v), v.stride(0), p(steps), p(decays), p(state), state.stride(0), n_offset, p(seg_q_start),
                     p(seg_q_len), p(state_slots), p(y), p(nq), bf(v), v.shape[0], seg_q_start.shape[0], heads, head_dim,
-                    value_dim, stream))
+                    value_dim, int(row_decays), stream))
     register_op("head_norm_gate", entry_point="wllm_head_norm_gate",
                 argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_float, c_int,
                           c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
                 launch=lambda fn, stream, y, gate, weight, out, heads, eps, activation, scale, nq=None, floor=None,
                 den_eps=0.0: fn(
-                    p(y), p(gate), gate.stride(0), p(weight), p(out), out.stride(0), p(nq), p(floor), den_eps, bf(gate),
-                    GATE_KINDS[activation], y.shape[0], heads, y.shape[1] // heads, eps, scale, stream))
+                    p(y), p(gate), gate.stride(0) if gate is not None else 0, p(weight), p(out), out.stride(0), p(nq), p(floor),
+                    den_eps, bf(out), GATE_KINDS[activation], y.shape[0], heads, y.shape[1] // heads, eps, scale, stream))
     register_op("moe_route", entry_point="wllm_moe_route",
                 argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
-                          c_void_p],
-                launch=lambda fn, stream, x, router, ids, weights, groups, keep, eps: fn(
+                          c_int, c_int, c_void_p],
+                launch=lambda fn, stream, x, router, ids, weights, groups, keep, eps, scoring="softmax", normalize=True: fn(
                     p(x), p(router), p(ids), p(weights), bf(x), x.shape[0], x.shape[1], router.shape[0], ids.shape[1], groups,
-                    keep, eps, stream))
+                    keep, eps, MOE_SCORINGS[scoring], int(normalize), stream))
     register_op("moe_plan", entry_point="wllm_moe_plan", argtypes=[c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
                 launch=lambda fn, stream, ids, plan, experts, tile_rows=MOE_TILE_ROWS: fn(
                     p(ids), p(plan), ids.numel(), experts, moe_max_tiles(ids.numel(), experts, tile_rows), tile_rows, stream))
     register_op("moe_experts_up", entry_point="wllm_moe_up",
                 argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                          c_void_p],
-                launch=lambda fn, stream, x, w, plan, act, top, activation, tiles=None, tile_rows=MOE_TILE_ROWS: fn(
+                          c_void_p, c_void_p],
+                launch=lambda fn, stream, x, w, plan, act, top, activation, tiles=None, tile_rows=MOE_TILE_ROWS,
+                in_weights=None: fn(
                     p(x), p(w), p(tiles), p(plan), moe_max_tiles(act.shape[0], w.shape[0], tile_rows), tile_rows, p(act), bf(x),
-                    ACTIVATIONS[activation], x.shape[1], act.shape[1], top, stream))
+                    ACTIVATIONS[activation], x.shape[1], act.shape[1], top, p(in_weights), stream))
     register_op("moe_experts_down", entry_point="wllm_moe_down",
                 argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                           c_int, c_void_p],
-                launch=lambda fn, stream, act, w, plan, weights, out, tiles=None, tile_rows=MOE_TILE_ROWS: fn(
-                    p(act), p(w), p(tiles), p(plan), moe_max_tiles(act.shape[0], w.shape[0], tile_rows), tile_rows, p(weights),
-                    p(out), bf(act), weights.shape[0], act.shape[1], w.shape[1], weights.shape[1], stream))
+                launch=lambda fn, stream, act, w, plan, weights, out, tiles=None, tile_rows=MOE_TILE_ROWS, weighted=True: fn(
+                    p(act), p(w), p(tiles), p(plan), moe_max_tiles(act.shape[0], w.shape[0], tile_rows), tile_rows,
+                    p(weights if weighted else None), p(out), bf(act), weights.shape[0], act.shape[1], w.shape[1], weights.shape[1], stream))
     tiles = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
              c_void_p]
     register_op("moe_experts_up_tiled", entry_point="wllm_moe_tiles", argtypes=tiles,
-                launch=lambda fn, stream, x, w, plan, act, top, activation: fn(
-                    p(x), p(w), p(plan), moe_max_tiles(act.shape[0], w.shape[0], MOE_BIG_TILE_ROWS), p(act), p(None), p(None),
+                launch=lambda fn, stream, x, w, plan, act, top, activation, in_weights=None: fn(
+                    p(x), p(w), p(plan), moe_max_tiles(act.shape[0], w.shape[0], MOE_BIG_TILE_ROWS), p(act), p(None), p(in_weights),
                     ACTIVATIONS[activation], x.shape[0], act.shape[1], x.shape[1], top, x.shape[0], stream))
     register_op("moe_experts_down_tiled", entry_point="wllm_moe_tiles", argtypes=tiles,
-                launch=lambda fn, stream, act, w, plan, weights, out: fn(
+                launch=lambda fn, stream, act, w, plan, weights, out, weighted=True: fn(
                     p(act), p(w), p(plan), moe_max_tiles(act.shape[0], w.shape[0], MOE_BIG_TILE_ROWS), p(None), p(out),
-                    p(weights), -1, act.shape[0], w.shape[1], act.shape[1], weights.shape[1], weights.shape[0], stream))
+                    p(weights if weighted else None), -1, act.shape[0], w.shape[1], act.shape[1], weights.shape[1], weights.shape[0], stream))
 
 _register_own()

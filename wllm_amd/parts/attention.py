@@ -20,6 +20,8 @@ the row and in the cache, with zeros that add nothing to a score or a result); a
 instead of a window; an RMS norm with a weight over the whole query projection and over the whole key
 projection (`ops.band_norm`) in place of the norm of each head; a gate of one number a head; and a
 layer without key and value projections that reads another layer's cache with its own queries.
+And: an RMS norm with a weight over every query head and every key head before the rotation (the weight
+has head_dim numbers that the heads share), and a learned number a head in the softmax's denominator.
 """
 from __future__ import annotations
 
@@ -47,7 +49,17 @@ class PagedAttention:
         plain = not (spec.softcap or spec.qk_norm_eps is not None or spec.values_are_keys or spec.gate_weight
                      or spec.position.pairing == "interleaved" or spec.value_dim not in (None, spec.head_dim)
                      or spec.chunk or spec.q_norm_weight or spec.k_norm_weight or not spec.owns_cache
-                     or spec.sink is not None or spec.output_scale != 1.0)
+                     or spec.sink is not None or spec.output_scale != 1.0 or spec.q_head_norm_weight
+                     or spec.k_head_norm_weight or spec.sink_weight or spec.position.magnitude != 1.0)
+        if bool(spec.q_head_norm_weight) != bool(spec.k_head_norm_weight) or (
+                spec.q_head_norm_weight and (spec.head_norm_eps is None or spec.head_norm_eps < 0)):
+            raise ValueError("a norm over each head has a weight for the queries, one for the keys, and head_norm_eps")
+        if spec.q_head_norm_weight and (spec.q_norm_weight or spec.k_norm_weight):
+            raise ValueError("a norm over each head and a norm over the whole projection: one of the two")
+        if spec.q_head_norm_weight and not spec.owns_cache:
+            raise ValueError("a norm over each head: the layer has keys of its own")
+        if spec.sink_weight and spec.sink is not None:
+            raise ValueError("sink and sink_weight: the denominator's term is a constant or a learned number a head")
         if spec.chunk is not None and (spec.chunk <= 0 or spec.window is not None):
             raise ValueError(f"chunk must be positive and excludes a window, got chunk {spec.chunk}, window {spec.window}")
         if (spec.q_norm_weight or spec.k_norm_weight) and spec.band_norm_eps is None:
@@ -87,6 +99,7 @@ class PagedAttention:
         if not 0 < self.dim <= ops.MAX_HEAD_DIM:
             raise ValueError(f"value_dim {self.vdim}: the attention kernels take heads up to {ops.MAX_HEAD_DIM}")
         self.w_q_norm = self.w_k_norm = None
+        self.w_q_head_norm = self.w_k_head_norm = None
         self.b_q = self.b_k = None          # biases that are added in front of the norm over a whole projection
         self.sinks = None
 
@@ -127,6 +140,11 @@ class PagedAttention:
             out[s.q_norm_weight] = ExpectedTensor((q,), role="vector", init="norm")
         if s.k_norm_weight and s.owns_cache:
             out[s.k_norm_weight] = ExpectedTensor((kv,), role="vector", init="norm")
+        if s.q_head_norm_weight:
+            out[s.q_head_norm_weight] = ExpectedTensor((s.head_dim,), role="vector", init="norm")
+            out[s.k_head_norm_weight] = ExpectedTensor((s.head_dim,), role="vector", init="norm")
+        if s.sink_weight:
+            out[s.sink_weight] = ExpectedTensor((s.num_heads,), role="vector", init="norm")
         for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, s.num_kv_heads * self.vdim), (s.o_bias, s.hidden_size)):
             if name is not None:
                 out[name] = ExpectedTensor((width,), role="vector")
@@ -188,6 +206,12 @@ class PagedAttention:
                 self.b_qkv = fetch.to_device(torch.cat(parts))
         if s.sink is not None:
             self.sinks = torch.full((s.num_heads,), float(s.sink), dtype=torch.float32, device=fetch.device)
+        if s.sink_weight:
+            self.sinks = fetch.to_device(fetch.vector(s.sink_weight))
+        if s.q_head_norm_weight:
+            # (a padded head's last elements are zero and stay zero under a weight of zero)
+            self.w_q_head_norm = fetch.to_device(heads_padded(fetch.vector(s.q_head_norm_weight), 0))
+            self.w_k_head_norm = fetch.to_device(heads_padded(fetch.vector(s.k_head_norm_weight), 0))
         if hasattr(self.position, "load"):
             self.position.load(fetch)
         self.position.prepare(fetch.device)
@@ -263,7 +287,7 @@ class PagedAttention:
                     qkv, self.b_qkv, ctx.positions, inv_freq, slots, storage, num_heads=s.num_heads,
                     num_kv_heads=s.num_kv_heads, head_dim=self.dim, page_size=pages.page_size,
                     interleaved=getattr(self.position, "interleaved", False), norm_eps=s.qk_norm_eps,
-                    values_are_keys=s.values_are_keys, norm_dim=s.head_dim)
+                    values_are_keys=s.values_are_keys, norm_dim=s.head_dim, rot_scale=getattr(self.position, "magnitude", 1.0))
         elif not self.plain:
             if apply is not None:
                 raise NotImplementedError("a position encoding with a step of its own beside the attention's options")
@@ -273,7 +297,8 @@ class PagedAttention:
                 num_kv_heads=s.num_kv_heads, head_dim=self.dim, page_size=pages.page_size,
                 interleaved=getattr(self.position, "interleaved", False), norm_eps=s.qk_norm_eps,
                 values_are_keys=s.values_are_keys, parts=projected if projected.dim() == 3 else None,
-                norm_dim=s.head_dim)
+                norm_dim=s.head_dim, rot_scale=getattr(self.position, "magnitude", 1.0),
+                head_norm=(self.w_q_head_norm, self.w_k_head_norm, s.head_norm_eps) if self.w_q_head_norm is not None else None)
         elif apply is not None:
             ops.linear(h, self.w_qkv, qkv, self.t_qkv)
             if self.b_qkv is not None:

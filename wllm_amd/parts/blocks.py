@@ -18,6 +18,12 @@ formed in the product's float32 accumulators, and the stream sees one contributi
 well as before it, then, if the layer has one, a per-layer token input that reads the stream itself.
 A sublayer's product stays pending together with the norm it has to pass (`pending_norm`), and the
 next norm kernel normalises it, adds it and normalises the sum for the next sublayer in one pass.
+
+"post_norm": x += post(mixer(x)); x += post(feed_forward(x)): no norm in front of a sublayer, which reads
+the stream itself, optionally through a short convolution over time (`InputConv`: the stream's value plus
+a weighted sum of its last few values, channel by channel).  The convolution's last inputs are state that
+the block, not its mixer, carries for a request: the block names it in `state_shapes()` and finds it
+under (run, name).
 """
 from __future__ import annotations
 
@@ -28,7 +34,8 @@ import torch
 from wllm_amd.kernels import ops
 from wllm_amd.parts.common import Product
 from wllm_amd.parts.registry import build_feed_forward, build_mixer, build_norm, register_block
-from wllm_amd.parts.specs import BlockSpec
+from wllm_amd.parts.specs import BlockSpec, InputConvSpec
+from wllm_amd.weights.checkpoint import ExpectedTensor
 
 
 class ResidualStream:
@@ -246,3 +253,83 @@ class SandwichBlock:
             stream.add(ctx, self.feed_forward.forward(ctx, h), norm=self.feed_forward_post_norm)
         if self.side is not None:
             stream.add(ctx, self.side.forward(ctx, stream.as_activations(ctx)), norm=self.side.norm)
+
+
+class InputConv:
+    """h_t + sum_j w[:, j] * h_(t - taps + 1 + j) on the residual stream, in float32, from the request's carried
+    rows (its last taps - 1 values of the stream; zeros for a fresh request, which are the zeros before a
+    sequence's start) and into them."""
+
+    def __init__(self, spec: InputConvSpec):
+        if spec.taps < 1 or spec.taps > 64 or spec.size <= 0:
+            raise ValueError(f"an input convolution has 1 to 64 taps over a positive number of channels, got {spec}")
+        self.spec = spec
+        self.weight = None
+
+    @property
+    def carried(self) -> int:
+        """Floats a request carries for this convolution."""
+        return (self.spec.taps - 1) * self.spec.size
+
+    def expected_tensors(self) -> dict:
+        return {self.spec.weight: ExpectedTensor((self.spec.size, self.spec.taps), role="vector")}
+
+    def load(self, fetch) -> None:
+        self.weight = fetch.to_device(fetch.vector(self.spec.weight))      # the taps stay float32
+
+    def forward(self, ctx, state: torch.Tensor, offset: int, stream: ResidualStream) -> torch.Tensor:
+        n, hidden = stream.x.shape
+        stream.settle()         # the convolution reads other tokens' rows of the stream: they take what is pending first
+        out = ctx.buffer("conv_in", (n, hidden), ctx.dtype)
+        ops.stream_conv(stream.x, self.weight, state, offset, ctx.token_segment, ctx.seg_q_start, ctx.seg_q_len,
+                        ctx.state_slots, out)
+        return out
+
+
+@register_block("post_norm")
+class PostNormBlock:
+    """x += post(mixer(read(x))); x += post(feed_forward(read(x))), read being the stream itself or its short
+    convolution over time."""
+    STATE = "input_conv"
+
+    def __init__(self, spec: BlockSpec):
+        if spec.mixer_norm is not None or spec.feed_forward_norm is not None:
+            raise ValueError("a post-norm block has no norm in front of a sublayer")
+        if spec.mixer_post_norm is None or (spec.feed_forward is not None and spec.feed_forward_post_norm is None):
+            raise ValueError("a post-norm block has a norm behind each of its sublayers")
+        if spec.feed_forward is None and spec.feed_forward_input_conv is not None:
+            raise ValueError("a convolution in front of a feed-forward that is not there")
+        self.spec = spec
+        self.mixer = build_mixer(spec.mixer)
+        self.mixer_post_norm = build_norm(spec.mixer_post_norm)
+        self.mixer_conv = InputConv(spec.mixer_input_conv) if spec.mixer_input_conv is not None else None
+        self.feed_forward = self.feed_forward_post_norm = self.feed_forward_conv = None
+        if spec.feed_forward is not None:
+            self.feed_forward = build_feed_forward(spec.feed_forward)
+            self.feed_forward_post_norm = build_norm(spec.feed_forward_post_norm)
+            if spec.feed_forward_input_conv is not None:
+                self.feed_forward_conv = InputConv(spec.feed_forward_input_conv)
+
+    def parts(self) -> list:
+        own = [self.mixer_conv, self.mixer, self.mixer_post_norm, self.feed_forward_conv, self.feed_forward,
+               self.feed_forward_post_norm]
+        return [p for p in own if p is not None]
+
+    def state_shapes(self) -> dict:
+        """The block's own state: the two convolutions' carried rows, the mixer's first."""
+        convs = [c for c in (self.mixer_conv, self.feed_forward_conv) if c is not None]
+        # (a convolution of one tap carries nothing, and still names a row)
+        return {self.STATE: (max(1, sum(c.carried for c in convs)),)} if convs else {}
+
+    def _read(self, ctx, entry: int, stream: ResidualStream, conv, offset: int) -> torch.Tensor:
+        if conv is None:
+            return stream.as_activations(ctx)
+        return conv.forward(ctx, ctx.state((entry, self.STATE)), offset, stream)
+
+    def forward(self, ctx, entry: int, stream: ResidualStream) -> None:
+        h = self._read(ctx, entry, stream, self.mixer_conv, 0)
+        stream.add(ctx, self.mixer.forward(ctx, entry, h), norm=self.mixer_post_norm)
+        if self.feed_forward is not None:
+            offset = self.mixer_conv.carried if self.mixer_conv is not None else 0
+            h = self._read(ctx, entry, stream, self.feed_forward_conv, offset)
+            stream.add(ctx, self.feed_forward.forward(ctx, h), norm=self.feed_forward_post_norm)

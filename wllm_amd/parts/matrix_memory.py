@@ -11,7 +11,12 @@ the two gate projections give a log input gate and a log forget gate (both bent 
 maximum m holds the exponentials in range, a normaliser n_t = a_t n_(t-1) + b_t k_t is carried beside S and
 den_t = max(|n_t . q_t|, exp(-m_t)) + den_eps (the matrix memory of an mLSTM).  The normaliser is one more
 column of the memory (a value that is always 1), so the recurrence's kernel carries it and leaves n . q beside
-the columns' sums; the kernel that norms the heads divides by den first.
+the columns' sums; the kernel that norms the heads divides by den first.  With "forget" there is no key
+projection: a forget gate a channel, f = l + (1 - l) sigmoid(W_f h + b) with a learned lower bound l, decays the
+rows of S and 1 - f stands in the key's place, S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T (the gating of HGRN2);
+the gate's projection lies where the keys' would in the stacked product, and the recurrence's kernel takes f as
+a decay a row.  Such a mixer may have no output gate, a silu on its queries, and a norm weight of value_dim
+numbers that its heads share.
 
 A request carries S (and n, m) from step to step in one float32 state row of the cache manager
 ([heads * head_dim * value_dim], then [heads * head_dim], then [heads]; zeroed at admission: all three
@@ -42,14 +47,24 @@ class MatrixMemoryMixer:
                 raise ValueError(f"{name} must be positive, got {getattr(spec, name)}")
         if spec.head_dim > 256:
             raise ValueError(f"head_dim {spec.head_dim}: the recurrence's kernel keeps at most 256 rows a head")
-        if spec.gating not in ("decay", "exponential"):
-            raise ValueError(f"gating {spec.gating!r}: 'decay' or 'exponential'")
+        if spec.gating not in ("decay", "exponential", "forget"):
+            raise ValueError(f"gating {spec.gating!r}: 'decay', 'exponential' or 'forget'")
+        if spec.gating == "forget" and (not spec.f_weight or spec.k_weight or spec.position.kind != "none"
+                                        or spec.q_scale != 1.0 or spec.k_scale != 1.0):
+            raise ValueError("forget gating: a forget projection, no key projection, no rotation and no scales")
+        if spec.gating != "forget" and (not spec.k_weight or not spec.gate_weight or spec.q_activation != "none"
+                                        or spec.lower_bound):
+            raise ValueError(f"gating {spec.gating!r} has key and gate projections and plain queries")
+        if spec.q_activation not in ops.QUERY_ACTIVATIONS:
+            raise ValueError(f"q_activation {spec.q_activation!r}: one of {sorted(ops.QUERY_ACTIVATIONS)}")
         if spec.gating == "decay" and len(spec.decays) != spec.num_heads:
             raise ValueError(f"decays: one a head ({spec.num_heads}), got {len(spec.decays)}")
         if spec.gating == "exponential" and not (spec.i_weight and spec.f_weight):
             raise ValueError("exponential gating needs the two gate projections")
         if spec.gate_cap is not None and not spec.gate_cap > 0:
             raise ValueError(f"gate_cap must be positive or None, got {spec.gate_cap}")
+        if spec.gate_weight and spec.gate_activation not in ("sigmoid", "silu"):
+            raise ValueError(f"gate_activation {spec.gate_activation!r}: 'sigmoid' or 'silu'")
         if spec.gate_activation not in ops.GATE_KINDS:
             raise ValueError(f"gate_activation {spec.gate_activation!r}: one of {sorted(ops.GATE_KINDS)}")
         if spec.position.kind == "rope" and (spec.position.pairing != "half" or spec.position.rotary_dim > spec.head_dim):
@@ -57,28 +72,37 @@ class MatrixMemoryMixer:
         self.spec = spec
         self.position = build_position(spec.position)
         self.exponential = spec.gating == "exponential"
+        self.forget = spec.gating == "forget"
         self.qk_width = spec.num_heads * spec.head_dim
         self.v_width = spec.num_heads * spec.value_dim
         self.v_offset = 2 * self.qk_width
         self.g_offset = self.v_offset + self.v_width
-        self.gates_offset = self.g_offset + self.v_width
+        self.gates_offset = self.g_offset + (self.v_width if spec.gate_weight else 0)
         width = self.gates_offset + (2 * spec.num_heads if self.exponential else 0)
         self.in_width = -(-width // 8) * 8             # rows of the stacked weight, padded with zero rows
         self.memory_size = spec.num_heads * spec.head_dim * spec.value_dim
         self.w_in = self.t_in = self.w_o = self.t_o = None
-        self.norm_w = self.i_bias = self.f_bias = self.decays = None
+        self.norm_w = self.i_bias = self.f_bias = self.decays = self.lower = None
 
     def expected_tensors(self) -> dict:
         s = self.spec
         out = {
             s.q_weight: ExpectedTensor((self.qk_width, s.hidden_size)),
-            s.k_weight: ExpectedTensor((self.qk_width, s.hidden_size)),
             s.v_weight: ExpectedTensor((self.v_width, s.hidden_size)),
-            s.gate_weight: ExpectedTensor((self.v_width, s.hidden_size)),
             s.o_weight: ExpectedTensor((s.hidden_size, self.v_width)),
         }
+        if s.gate_weight:
+            out[s.gate_weight] = ExpectedTensor((self.v_width, s.hidden_size))
+        if self.forget:
+            out[s.f_weight] = ExpectedTensor((self.qk_width, s.hidden_size))
+            for name in (s.f_bias, s.lower_bound):
+                if name:
+                    out[name] = ExpectedTensor((self.qk_width,), role="vector")
+        else:
+            out[s.k_weight] = ExpectedTensor((self.qk_width, s.hidden_size))
         if s.norm_weight:
-            out[s.norm_weight] = ExpectedTensor((self.v_width,), role="vector", init="norm")
+            out[s.norm_weight] = ExpectedTensor((self.v_width if s.norm_weight_per_head else s.value_dim,), role="vector",
+                                                init="norm")
         if self.exponential:
             out[s.i_weight] = ExpectedTensor((s.num_heads, s.hidden_size))
             out[s.f_weight] = ExpectedTensor((s.num_heads, s.hidden_size))
@@ -89,7 +113,10 @@ class MatrixMemoryMixer:
 
     def load(self, fetch) -> None:
         s = self.spec
-        stacked = [fetch.matrix(name) for name in (s.q_weight, s.k_weight, s.v_weight, s.gate_weight)]
+        # (with forget gating the gate's projection lies where the keys' would)
+        stacked = [fetch.matrix(name) for name in (s.q_weight, s.f_weight if self.forget else s.k_weight, s.v_weight)]
+        if s.gate_weight:
+            stacked.append(fetch.matrix(s.gate_weight))
         if self.exponential:
             stacked += [fetch.matrix(s.i_weight), fetch.matrix(s.f_weight)]
         w = torch.cat(stacked, dim=0)
@@ -99,8 +126,12 @@ class MatrixMemoryMixer:
         self.w_o, self.t_o = load_matrix(fetch, fetch.matrix(s.o_weight))
         # everything that enters the recurrence is kept in float32
         if s.norm_weight:
-            self.norm_w = fetch.to_device(fetch.vector(s.norm_weight))
-        if self.exponential:
+            norm_w = fetch.vector(s.norm_weight)
+            self.norm_w = fetch.to_device(norm_w if s.norm_weight_per_head else norm_w.repeat(s.num_heads))
+        if self.forget:
+            self.f_bias = fetch.to_device(fetch.vector(s.f_bias)) if s.f_bias else None
+            self.lower = fetch.to_device(fetch.vector(s.lower_bound)) if s.lower_bound else None
+        elif self.exponential:
             self.i_bias = fetch.to_device(fetch.vector(s.i_bias)) if s.i_bias else None
             self.f_bias = fetch.to_device(fetch.vector(s.f_bias)) if s.f_bias else None
         else:
@@ -124,10 +155,14 @@ class MatrixMemoryMixer:
         row = ctx.buffer("memory_in", (n, self.in_width), h.dtype)
         ops.linear(h, self.w_in, row, self.t_in)
         state = ctx.state(entry)
-        qk = ctx.buffer("memory_qk", (2, n, self.qk_width), torch.float32)
-        ops.memory_inputs(row, ctx.positions, self.position.inv_freq, qk, heads=s.num_heads, head_dim=s.head_dim,
-                          q_scale=s.q_scale, k_scale=s.k_scale)
         steps = nq = None
+        if self.forget:
+            qk = ctx.buffer("memory_qkf", (3, n, self.qk_width), torch.float32)
+            ops.memory_forget_inputs(row, self.f_bias, self.lower, qk, width=self.qk_width, q_activation=s.q_activation)
+        else:
+            qk = ctx.buffer("memory_qk", (2, n, self.qk_width), torch.float32)
+            ops.memory_inputs(row, ctx.positions, self.position.inv_freq, qk, heads=s.num_heads, head_dim=s.head_dim,
+                              q_scale=s.q_scale, k_scale=s.k_scale)
         if self.exponential:
             # the normaliser lies behind the memory in the request's row, the running maxima behind it
             n_offset = self.memory_size
@@ -139,9 +174,11 @@ class MatrixMemoryMixer:
         y = ctx.buffer("memory_y", (n, self.v_width), torch.float32)
         ops.memory_scan(qk, row[:, self.v_offset:self.v_offset + self.v_width], steps, self.decays, state,
                         ctx.seg_q_start, ctx.seg_q_len, ctx.state_slots, y, heads=s.num_heads, head_dim=s.head_dim,
-                        value_dim=s.value_dim, nq=nq, n_offset=self.memory_size if self.exponential else 0)
+                        value_dim=s.value_dim, nq=nq, n_offset=self.memory_size if self.exponential else 0,
+                        row_decays=self.forget)
         out = product_input if product_input is not None else ctx.buffer("memory_out", (n, self.v_width), h.dtype)
-        ops.head_norm_gate(y, row[:, self.g_offset:self.g_offset + self.v_width], self.norm_w, out, heads=s.num_heads,
-                           eps=s.norm_eps, activation=s.gate_activation, scale=s.output_scale, nq=nq,
+        gate = row[:, self.g_offset:self.g_offset + self.v_width] if s.gate_weight else None
+        ops.head_norm_gate(y, gate, self.norm_w, out, heads=s.num_heads,
+                           eps=s.norm_eps, activation=s.gate_activation if s.gate_weight else "none", scale=s.output_scale, nq=nq,
                            floor=steps[2] if self.exponential else None, den_eps=s.den_eps if self.exponential else 0.0)
         return Product("mixer_out", out, self.w_o, self.t_o)

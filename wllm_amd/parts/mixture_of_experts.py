@@ -14,12 +14,19 @@ memory where they get many (a prompt's portion).  The second product weighs a pa
 leaves it in the slice of its slot of a float32 stack [top, tokens, width], which whoever adds the
 feed-forward to the stream (the next norm kernel) adds in order: the weighted sum is formed in float32
 and takes no pass of its own.  Nothing of the routing is read on the host.
+
+Options: the scores may be sigmoids of the logits, every expert by itself (`scoring`), and the chosen scores
+may be the weights as they are (`normalize` False); the weight may multiply the expert's input instead of its
+output (`weight_on_input`: the factor is taken out of the first product's two sums and multiplied in before the
+activation, and the second product's results are not weighed); and one more gated feed-forward may run for
+every token (`shared`), whose result is one more slice of the stack.
 """
 from __future__ import annotations
 
 import torch
 
 from wllm_amd.kernels import ops
+from wllm_amd.parts.feed_forward import GatedMLP
 from wllm_amd.parts.registry import register_feed_forward
 from wllm_amd.parts.specs import MixtureOfExpertsSpec
 from wllm_amd.weights.checkpoint import ExpectedTensor
@@ -39,7 +46,10 @@ class MixtureOfExperts:
                              f"keep_groups ({spec.keep_groups}) lie between 1 and num_groups")
         if not 0 < spec.top <= spec.keep_groups * (spec.num_experts // spec.num_groups):
             raise ValueError(f"top ({spec.top}): at most the experts of the kept groups")
+        if spec.scoring not in ops.MOE_SCORINGS:
+            raise ValueError(f"scoring {spec.scoring!r}: one of {sorted(ops.MOE_SCORINGS)}")
         self.spec = spec
+        self.shared = GatedMLP(spec.shared) if spec.shared is not None else None
         self.w_router = self.w_up = self.w_down = None
         self.t_up = self.t_down = None          # the stacks' tile-major copies, which the few-row kernels stream
 
@@ -57,10 +67,17 @@ class MixtureOfExperts:
             out[gate] = ExpectedTensor((s.intermediate_size, s.hidden_size))
             out[up] = ExpectedTensor((s.intermediate_size, s.hidden_size))
             out[down] = ExpectedTensor((s.hidden_size, s.intermediate_size))
+        if self.shared is not None:
+            out.update(self.shared.expected_tensors())
         return out
+
+    def sub_parts(self) -> tuple:
+        return (self.shared,) if self.shared is not None else ()
 
     def load(self, fetch) -> None:
         s = self.spec
+        if self.shared is not None:
+            self.shared.load(fetch)
         ups, downs = [], []
         for e in range(s.num_experts):
             gate, up, down = self._names(e)
@@ -77,7 +94,8 @@ class MixtureOfExperts:
 
     def flops(self, tokens: int) -> float:
         s = self.spec
-        return 2.0 * tokens * s.hidden_size * (3 * s.top * s.intermediate_size + s.num_experts)
+        shared = self.shared.flops(tokens) if self.shared is not None else 0.0
+        return 2.0 * tokens * s.hidden_size * (3 * s.top * s.intermediate_size + s.num_experts) + shared
 
     def bytes_read(self, tokens: int) -> float:
         """Bytes of expert weights a step of `tokens` tokens reads if the router spreads the tokens evenly: every
@@ -93,12 +111,18 @@ class MixtureOfExperts:
         n = h.shape[0]
         ids = ctx.buffer("moe_ids", (n, s.top), torch.int32)
         weights = ctx.buffer("moe_weights", (n, s.top), torch.float32)
-        ops.moe_route(h, self.w_router, ids, weights, groups=s.num_groups, keep=s.keep_groups, eps=s.weight_eps)
+        ops.moe_route(h, self.w_router, ids, weights, groups=s.num_groups, keep=s.keep_groups, eps=s.weight_eps,
+                      scoring=s.scoring, normalize=s.normalize)
         rows = ops.moe_tile_rows(n * s.top, s.num_experts, h.dtype, s.hidden_size, s.intermediate_size)
         plan = ctx.buffer("moe_plan", (ops.moe_plan_size(n * s.top, s.num_experts, rows),), torch.int32)
         ops.moe_plan(ids, plan, s.num_experts, rows)
         act = ctx.buffer("moe_act", (n * s.top, s.intermediate_size), h.dtype)
-        ops.moe_experts_up(h, self.w_up, plan, act, s.top, s.activation, rows, self.t_up)
-        out = ctx.buffer("moe_out", (s.top, n, s.hidden_size), torch.float32)
-        ops.moe_experts_down(act, self.w_down, plan, weights, out, rows, self.t_down)
+        ops.moe_experts_up(h, self.w_up, plan, act, s.top, s.activation, rows, self.t_up,
+                           in_weights=weights if s.weight_on_input else None)
+        out = ctx.buffer("moe_out", (s.top + (1 if self.shared is not None else 0), n, s.hidden_size), torch.float32)
+        ops.moe_experts_down(act, self.w_down, plan, weights, out[:s.top], rows, self.t_down, weighted=not s.weight_on_input)
+        if self.shared is not None:
+            # the expert every token uses: its product's float32 sums are the stack's last slice
+            last = self.shared.forward(ctx, h)
+            ops.linear(last.x, last.weight, out[s.top], last.tiles)
         return out

@@ -69,9 +69,13 @@ class CausalLM:
     def state_shapes(self) -> dict:
         shapes = {}
         for i, e in enumerate(self.plan.schedule):
-            shape = self.blocks[e.layer].mixer.state_shape()      # a shape (float32) or a StateNeed
+            block = self.blocks[e.layer]
+            shape = block.mixer.state_shape()      # a shape (float32) or a StateNeed
             if shape is not None:
                 shapes[i] = shape
+            # what the block itself carries for a request beside its mixer's state, under (run, name)
+            for name, own in getattr(block, "state_shapes", dict)().items():
+                shapes[(i, name)] = own
         return shapes
 
     def graph_capturable(self) -> bool:
@@ -191,6 +195,8 @@ class CausalLM:
         last = stream.normed(self.final_norm, ctx.buffer("final_normed", (m, hidden), self.dtype), rows=ctx.logit_rows)
         logits = ctx.buffer("logits", (m, vocab), torch.float32)
         ops.linear(last, self.head_weight, logits, self.head_tiles)
+        if self.plan.head.logit_scale != 1.0:
+            ops.copy_columns(logits, logits, self.plan.head.logit_scale)
         return logits
 
 

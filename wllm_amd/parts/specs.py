@@ -29,12 +29,20 @@ class PositionSpec:
     """How positions enter a mixer.  kind "rope": rotation of query and key by
     angles position * theta^(-2j/rotary_dim) / scaling_factor, pairing element j with
     j + rotary_dim/2 ("half") or element 2j with 2j + 1 ("interleaved"); elements of a head
-    beyond rotary_dim pass unchanged.  kind "none": nothing."""
+    beyond rotary_dim pass unchanged.  kind "none": nothing.
+    `ramp` = (factor, original, fast, slow) interpolates the frequencies pair by pair between their plain values
+    and those divided by `factor`: with pair(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta),
+    lo = max(floor(pair(fast)), 0), hi = min(ceil(pair(slow)), rotary_dim - 1) and
+    r_j = clamp((j - lo) / max(hi - lo, 0.001), 0, 1), pair j turns by f_j / factor * r_j + f_j * (1 - r_j): pairs
+    that make many turns within `original` positions keep their frequency, slow ones are stretched.
+    `magnitude`: sine and cosine are both multiplied by it."""
     kind: str = "rope"
     rotary_dim: int = 0
     theta: float = 10000.0
     pairing: str = "half"
     scaling_factor: float = 1.0     # linear scaling: every frequency is divided by it
+    ramp: Optional[tuple] = None
+    magnitude: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -70,7 +78,11 @@ class AttentionSpec(MixerSpec):
     every head, a term with no key and no value (0.0: one is added to the sum of exponentials).
     `bias_before_norm`: the biases of the query and key projections are added before the norm over the
     whole projection, not behind it.  `output_scale`: the concatenated heads are multiplied by it before
-    the output projection (a mixer whose result enters a weighted sum with another's)."""
+    the output projection (a mixer whose result enters a weighted sum with another's).
+    `q_head_norm_weight` / `k_head_norm_weight` with `head_norm_eps`: before the rotation every query head and
+    every key head passes an RMS norm over its own elements with a weight of head_dim numbers that the heads
+    share.  `sink_weight`: the term in the softmax's denominator is exp(sink_h) of a learned number a head
+    (a tensor [num_heads]) instead of the constant `sink`."""
     kind: str = "attention"
     hidden_size: int = 0
     num_heads: int = 0
@@ -103,6 +115,10 @@ class AttentionSpec(MixerSpec):
     sink: Optional[float] = None
     bias_before_norm: bool = False
     output_scale: float = 1.0
+    q_head_norm_weight: Optional[str] = None
+    k_head_norm_weight: Optional[str] = None
+    head_norm_eps: Optional[float] = None
+    sink_weight: Optional[str] = None
 
 
 @dataclass(frozen=True)
@@ -111,7 +127,13 @@ class LatentAttentionSpec(MixerSpec):
     (`kv_rank` numbers, the only thing cached), without positions: c_q = rms(W_dq h) * w_dqn, q = W_uq c_q;
     c = rms(W_dkv h) * w_dkvn; per head k = W_uk c, v = W_uv c; score = q.k * scale; with `sink_weight` the
     softmax's denominator holds exp(sink_h) once more; the concatenated heads are multiplied by
-    sigmoid(W_g h) and projected by W_o."""
+    sigmoid(W_g h) and projected by W_o.
+    `q_weight` (then `q_rank` is 0 and the three tensors of the queries' latent are not named): q = W_q h.
+    `rope_dim` r > 0 with `position`: a query head is [head_dim elements | r elements], W_dkv has kv_rank + r rows of
+    which the last r (not normed) are one more part of the key that all heads share; the r elements of the query heads
+    and of that key part turn by the position, and the score is (q . k + q_r . k_r) * scale.  Cached: c and the turned
+    key part.  `gate_weight` None: no gate.  `weights_in_float32`: the softmax weights are not rounded to the values' type
+    before they weigh the values."""
     kind: str = "latent_attention"
     hidden_size: int = 0
     num_heads: int = 0
@@ -131,6 +153,10 @@ class LatentAttentionSpec(MixerSpec):
     sink_weight: Optional[str] = None
     gate_weight: Optional[str] = None
     o_weight: str = ""
+    q_weight: Optional[str] = None
+    rope_dim: int = 0
+    position: PositionSpec = field(default_factory=lambda: PositionSpec(kind="none"))
+    weights_in_float32: bool = False
 
 
 @dataclass(frozen=True)
@@ -172,7 +198,12 @@ class MatrixMemorySpec(MixerSpec):
     n_t = a_t n_(t-1) + b_t k_t; den_t = max(|n_t . q_t|, exp(-m_t)) + `den_eps` (the matrix memory of an mLSTM).
     Then every head's o is divided by its root mean square (`norm_eps` inside the root), the heads are
     concatenated, multiplied by `norm_weight` (if named), by act(W_g h) with `gate_activation` "sigmoid" or
-    "silu", by `output_scale`, and projected by W_o.  A request carries S (and n, m) from token to token."""
+    "silu", by `output_scale`, and projected by W_o.  A request carries S (and n, m) from token to token.
+    `gating` "forget": a forget gate a channel that also decides what is written (HGRN2).  There is no key
+    projection: f = l + (1 - l) * sigmoid(W_f h + b_f) with a lower bound l a channel (`lower_bound`, a tensor
+    [heads * head_dim]; not named: 0), S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T, den_t = 1; f multiplies the
+    rows of S, those of q's channels.  `q_activation` "silu": q = silu(W_q h).  `gate_weight` None: no gate
+    behind the norm.  `norm_weight_per_head` False: `norm_weight` has value_dim numbers that the heads share."""
     kind: str = "matrix_memory"
     hidden_size: int = 0
     num_heads: int = 0
@@ -198,6 +229,9 @@ class MatrixMemorySpec(MixerSpec):
     i_bias: Optional[str] = None
     f_weight: Optional[str] = None
     f_bias: Optional[str] = None
+    lower_bound: Optional[str] = None
+    q_activation: str = "none"
+    norm_weight_per_head: bool = True
 
 
 @dataclass(frozen=True)
@@ -252,7 +286,10 @@ class MixtureOfExpertsSpec(FeedForwardSpec):
     `keep_groups` best groups can be chosen (one group, one kept: no limit).  The `top` allowed experts with
     the largest s are chosen, their weights are their s divided by the sum of the chosen (+ `weight_eps`),
     and the result is the weighted sum of their outputs.  `expert_prefix` + "<e>." + `gate_name` ... name an
-    expert's tensors."""
+    expert's tensors.  `scoring` "sigmoid": s = sigmoid(z), every expert by itself.  `normalize` False: the
+    weights are the chosen s themselves.  `weight_on_input`: the weight multiplies the expert's input instead of
+    its output, y = sum of expert_e(w_e x).  `shared`: one more gated feed-forward that every token uses, added to
+    the experts' sum."""
     kind: str = "mixture_of_experts"
     hidden_size: int = 0
     intermediate_size: int = 0
@@ -267,6 +304,20 @@ class MixtureOfExpertsSpec(FeedForwardSpec):
     gate_name: str = "gate"
     up_name: str = "up"
     down_name: str = "down"
+    scoring: str = "softmax"
+    normalize: bool = True
+    weight_on_input: bool = False
+    shared: Optional[GatedMLPSpec] = None
+
+
+@dataclass(frozen=True)
+class InputConvSpec:
+    """A short causal convolution over time on each channel of what a sublayer reads: h_t becomes
+    h_t + sum_j w[:, j] * h_(t - taps + 1 + j) with zeros before the sequence's start; `weight` [size, taps],
+    no bias.  A request carries its last taps - 1 inputs."""
+    size: int
+    taps: int
+    weight: str
 
 
 @dataclass(frozen=True)
@@ -277,15 +328,20 @@ class BlockSpec:
     sublayers read it (`feed_forward_norm` is None, and `feed_forward` may be None: then the
     layer is its mixer alone).  "sandwich": x += post(mixer(pre(x))); x += post(ffn(pre(x))) with the
     two norms behind the sublayers in `mixer_post_norm` and `feed_forward_post_norm` (a layer without a
-    feed-forward has neither of its norms), then the layer's token input (`side`), if it has one."""
+    feed-forward has neither of its norms), then the layer's token input (`side`), if it has one.
+    "post_norm": x += post(mixer(x)); x += post(ffn(x)): the sublayers read the stream itself and the only norms
+    stand behind them (`mixer_norm` and `feed_forward_norm` are None).  With `mixer_input_conv` /
+    `feed_forward_input_conv` what a sublayer reads first passes a short convolution over time (`InputConvSpec`)."""
     mixer: MixerSpec
     feed_forward: Optional[FeedForwardSpec]
-    mixer_norm: NormSpec
+    mixer_norm: Optional[NormSpec]
     feed_forward_norm: Optional[NormSpec]
     arrangement: str = "pre_norm"
     mixer_post_norm: Optional[NormSpec] = None
     feed_forward_post_norm: Optional[NormSpec] = None
     side: Optional[TokenSideSpec] = None
+    mixer_input_conv: Optional[InputConvSpec] = None
+    feed_forward_input_conv: Optional[InputConvSpec] = None
 
 
 @dataclass(frozen=True)
@@ -303,11 +359,12 @@ class EmbeddingSpec:
 class HeadSpec:
     """logits = hidden @ W^T; W is the embedding table when `weight` is None.  `tied_checkpoint_name`:
     the name under which a checkpoint of tied weights may still store the head; such a tensor is
-    accepted if it equals the table."""
+    accepted if it equals the table.  `logit_scale`: the logits are multiplied by it (in float32)."""
     vocab_size: int
     hidden_size: int
     weight: Optional[str] = None
     tied_checkpoint_name: Optional[str] = None
+    logit_scale: float = 1.0
 
 
 @dataclass(frozen=True)
