@@ -140,23 +140,25 @@ def forget_gate_recurrence(h, w, p, c, eps, rounding=same):
 def latent_attention(h, w, p, c, eps, rounding=same):
     """The "latent_attention" mixer."""
     T = h.shape[0]
-    H, d, dr, dv, rank = c["heads"], c["dim"], c["rot_dim"], c["vdim"], c["kv_rank"]
+    H, d, dr, dv, rank = c["heads"], c["dim"], c.get("rot_dim", 0), c["vdim"], c["kv_rank"]
     q = rounding(h @ w[p + "q"].T).view(T, H, d + dr)
     down = rounding(h @ w[p + "dkv"].T)
     latent = rounding(rms_norm(down[:, :rank], w[p + "dkv.norm"], eps))
     k_turned = down[:, rank:].view(T, 1, dr)
     k_plain = rounding(latent @ w[p + "uk"].T).view(T, H, d)
     v = rounding(latent @ w[p + "uv"].T).view(T, H, dv)
-    rot = c["rot"]
-    if rot.get("scaling"):
-        freq, magnitude = interpolated_frequencies(rot["dims"], rot["base"], rot["scaling"])
-    else:
-        freq, magnitude = plain_frequencies(rot["dims"], rot["base"]), 1.0
-    pos = torch.arange(T)
-    q_turned = rounding(rotate(q[..., d:], pos, rot["dims"], freq, "interleaved", magnitude))
-    k_turned = rounding(rotate(k_turned, pos, rot["dims"], freq, "interleaved", magnitude))
-    scores = (torch.einsum("thd,shd->hts", q[..., :d], k_plain)
-              + torch.einsum("thd,sd->hts", q_turned, k_turned[:, 0])) * c["scale"]
+    scores = torch.einsum("thd,shd->hts", q[..., :d], k_plain)
+    if dr:          # a model may have no turned part
+        rot = c["rot"]
+        if rot.get("scaling"):
+            freq, magnitude = interpolated_frequencies(rot["dims"], rot["base"], rot["scaling"])
+        else:
+            freq, magnitude = plain_frequencies(rot["dims"], rot["base"]), 1.0
+        pos = torch.arange(T)
+        q_turned = rounding(rotate(q[..., d:], pos, rot["dims"], freq, "interleaved", magnitude))
+        k_turned = rounding(rotate(k_turned, pos, rot["dims"], freq, "interleaved", magnitude))
+        scores = scores + torch.einsum("thd,sd->hts", q_turned, k_turned[:, 0])
+    scores = scores * c["scale"]
     weights = causal_softmax(scores)
     o = torch.einsum("hts,shd->thd", weights, v)
     return rounding(o.reshape(T, H * dv)) @ w[p + "o"].T
@@ -172,10 +174,11 @@ def sink_attention(h, w, p, c, eps, rounding=same):
     gate = rounding(h @ w[p + "g"].T)
     q = rms_norm(q, w[p + "q.norm"], eps)
     k = rms_norm(k, w[p + "k.norm"], eps)
-    rot = c["rot"]
-    freq, pos = plain_frequencies(rot["dims"], rot["base"]), torch.arange(T)
-    q = rounding(rotate(q, pos, rot["dims"], freq, "half"))
-    k = rounding(rotate(k, pos, rot["dims"], freq, "half"))
+    rot = c.get("rot")
+    if rot is not None:
+        freq, pos = plain_frequencies(rot["dims"], rot["base"]), torch.arange(T)
+        q, k = rotate(q, pos, rot["dims"], freq, "half"), rotate(k, pos, rot["dims"], freq, "half")
+    q, k = rounding(q), rounding(k)
     k = k.repeat_interleave(H // G, dim=1)
     v = v.repeat_interleave(H // G, dim=1)
     scores = torch.einsum("thd,shd->hts", q, k) * c["scale"]
