@@ -266,7 +266,7 @@ def main() -> int:
     ap.add_argument("--workload", default="decode", choices=["decode", "stress", "compare"],
                     help="decode: the contract's line; stress: continuous batching of 64 mixed requests; compare: prefill "
                          "and decode of the pairs of shapes of --compare, one model after the other")
-    ap.add_argument("--compare", default="tasosun-2b:gemma-2b,tasosun-7b:gemma-7b",   # also: tokuvik-2b:gemma-2b, lefisun-2b:tokuvik-2b
+    ap.add_argument("--compare", default="tasosun-2b:gemma-2b,tasosun-7b:gemma-7b",   # also: tokuvik-2b:gemma-2b, lefisun-2b:tokuvik-2b, duvozen-2b:tokuvik-2b
                     help="compare: pairs of shapes (named, or config.json files), new:closest, with commas between pairs")
     ap.add_argument("--stress-requests", type=int, default=64)
     ap.add_argument("--row-multiple", type=int, default=256,

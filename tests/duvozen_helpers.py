@@ -136,7 +136,7 @@ def random_config(seed: int) -> dict:
     """A configuration drawn from what the design allows: any order of mixers, any sizes."""
     import random
     r = random.Random(seed)
-    width = r.choice([32, 48, 64, 80])
+    width = r.choice([32, 48, 64, 80, 72, 100])
 
     def draw_mlp():
         u = r.random()

@@ -124,5 +124,10 @@ class MixtureOfExperts:
         if self.shared is not None:
             # the expert every token uses: its product's float32 sums are the stack's last slice
             last = self.shared.forward(ctx, h)
-            ops.linear(last.x, last.weight, out[s.top], last.tiles)
+            if h.dtype == torch.float32 or n <= 64:
+                ops.linear(last.x, last.weight, out[s.top], last.tiles)
+            else:
+                # many rows: the product as every other of this size is made (in the activation type), then into its slice
+                out[s.top].zero_()
+                ops.stream_add(out[s.top], delta=last.make(ctx))
         return out
