@@ -306,9 +306,11 @@ class EmulatedKernels:
             if taps > 1:
                 carried.copy_(seq[ql:].to(torch.float32))
 
-    def stream_conv(self, x, weight, state, carried_offset, token_segment, seg_q_start, seg_q_len, state_slots, out):
+    def stream_conv(self, x, weight, state, carried_offset, token_segment, seg_q_start, seg_q_len, state_slots, out,
+                    single_tokens=False):
         self._count("stream_conv")
-        c, taps = weight.shape
+        assert not single_tokens or all(int(n) == 1 for n in seg_q_len)
+        taps, c = weight.shape
         for s in range(seg_q_start.shape[0]):
             q0, ql, slot = int(seg_q_start[s]), int(seg_q_len[s]), int(state_slots[s])
             if ql == 0:
@@ -317,7 +319,7 @@ class EmulatedKernels:
             seq = torch.cat([carried.to(self.acc), x[q0:q0 + ql].to(self.acc)], dim=0)
             acc = x[q0:q0 + ql].to(self.acc).clone()
             for k in range(taps):
-                acc = acc + seq[k:k + ql] * weight[:, k].to(self.acc)
+                acc = acc + seq[k:k + ql] * weight[k].to(self.acc)
             out[q0:q0 + ql] = acc.to(out.dtype)
             if taps > 1:
                 carried.copy_(seq[ql:ql + taps - 1].float())

@@ -84,47 +84,119 @@ WLLM_API int wllm_causal_conv(const void* in, long long in_stride, const float* 
 }
 
 // ---- the same convolution on the residual stream itself, in front of a sublayer that reads the stream:
-// out[t, c] = x[t, c] + sum_k w[c, k] * x[t - (taps - 1) + k, c], float32 sums in this order, no bias and no
+// out[t, c] = x[t, c] + sum_k w[k, c] * x[t - (taps - 1) + k, c] (w a row a tap, [taps, channels]), float32 sums in this order, no bias and no
 // activation; x float32 [tokens, channels], out the activation type.  The carried rows (the request's last
-// taps - 1 rows of x, the oldest first) are kept by `conv_carry_kernel`, as above. ----
-template <typename T>
+// taps - 1 rows of x, the oldest first) are kept by `conv_carry_kernel`, as above; or, CARRY (a step of single
+// tokens, where no other token of the launch reads a request's carried rows), by the token's own threads, each
+// moving its channel's rows up by one as it reads them: one launch instead of two, the same sums. ----
+template <typename T, bool CARRY>
 __global__ void __launch_bounds__(256)
-stream_conv_kernel(const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ state,
+stream_conv_kernel(const float* __restrict__ x, const float* __restrict__ weight, float* __restrict__ state,
                    long long state_stride, long long carried_offset, const int* __restrict__ token_segment,
                    const int* __restrict__ seg_q_start, const int* __restrict__ state_slots, T* __restrict__ out,
                    int channels, int taps) {
     const int token = blockIdx.x;
     const int seg = token_segment[token];
     const int local = token - seg_q_start[seg];
-    const float* carried = state + static_cast<size_t>(state_slots[seg]) * state_stride + carried_offset;
+    float* carried = state + static_cast<size_t>(state_slots[seg]) * state_stride + carried_offset;
     for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
         float acc = x[static_cast<size_t>(token) * channels + c];
+        if (CARRY) {
+            // the segment is this one token: every earlier input is a carried row
+            const float now = acc;
+            for (int k = 0; k + 1 < taps; ++k) {
+                const float v = carried[static_cast<size_t>(k) * channels + c];
+                acc = fmaf(weight[static_cast<size_t>(k) * channels + c], v, acc);
+                if (k > 0) carried[static_cast<size_t>(k - 1) * channels + c] = v;
+            }
+            acc = fmaf(weight[static_cast<size_t>(taps - 1) * channels + c], now, acc);
+            if (taps > 1) carried[static_cast<size_t>(taps - 2) * channels + c] = now;
+            out[static_cast<size_t>(token) * channels + c] = from_float<T>(acc);
+            continue;
+        }
         for (int k = 0; k < taps; ++k) {
             const int src = local - (taps - 1) + k;
             const float v = src >= 0 ? x[static_cast<size_t>(token - local + src) * channels + c]
                                      : carried[static_cast<size_t>(taps - 1 + src) * channels + c];
-            acc = fmaf(weight[static_cast<size_t>(c) * taps + k], v, acc);
+            acc = fmaf(weight[static_cast<size_t>(k) * channels + c], v, acc);
         }
         out[static_cast<size_t>(token) * channels + c] = from_float<T>(acc);
+    }
+}
+
+// The same sums, four consecutive channels a thread with 16-byte loads of x and of the carried rows (a prompt's
+// portion: the kernel is bound by what it moves).  Channels, the carried rows' offset and the state's row are
+// multiples of four floats.
+template <typename T> struct alignas(4 * sizeof(T)) ConvFour { T v[4]; };
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+stream_conv_four_kernel(const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ state,
+                        long long state_stride, long long carried_offset, const int* __restrict__ token_segment,
+                        const int* __restrict__ seg_q_start, const int* __restrict__ state_slots, T* __restrict__ out,
+                        int channels, int taps) {
+    const int token = blockIdx.x;
+    const int seg = token_segment[token];
+    const int local = token - seg_q_start[seg];
+    const float* carried = state + static_cast<size_t>(state_slots[seg]) * state_stride + carried_offset;
+    for (int c = (blockIdx.y * blockDim.x + threadIdx.x) * 4; c < channels; c += gridDim.y * blockDim.x * 4) {
+        const float4 now = *reinterpret_cast<const float4*>(x + static_cast<size_t>(token) * channels + c);
+        float acc[4] = {now.x, now.y, now.z, now.w};
+        for (int k = 0; k < taps; ++k) {
+            const int src = local - (taps - 1) + k;
+            const float4 v = *reinterpret_cast<const float4*>(
+                src >= 0 ? x + static_cast<size_t>(token - local + src) * channels + c
+                         : carried + static_cast<size_t>(taps - 1 + src) * channels + c);
+            const float4 w = *reinterpret_cast<const float4*>(weight + static_cast<size_t>(k) * channels + c);
+            acc[0] = fmaf(w.x, v.x, acc[0]);
+            acc[1] = fmaf(w.y, v.y, acc[1]);
+            acc[2] = fmaf(w.z, v.z, acc[2]);
+            acc[3] = fmaf(w.w, v.w, acc[3]);
+        }
+        ConvFour<T> r;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) r.v[u] = from_float<T>(acc[u]);
+        *reinterpret_cast<ConvFour<T>*>(out + static_cast<size_t>(token) * channels + c) = r;
     }
 }
 
 WLLM_API int wllm_stream_conv(const float* x, const float* weight, float* state, long long state_stride,
                               long long carried_offset, const int* token_segment, const int* seg_q_start,
                               const int* seg_q_len, const int* state_slots, void* out, int out_bf16, int tokens,
-                              int segments, int channels, int taps, hipStream_t stream) {
+                              int segments, int channels, int taps, int single_tokens, hipStream_t stream) {
     if (tokens <= 0 || segments <= 0) return 0;
     if (channels <= 0 || taps < 1 || taps > 64) return -1;
+    if (single_tokens && tokens != segments) return -1;      // `single_tokens`: every segment is one token
     const int tiles = (channels + 255) / 256 < 64 ? (channels + 255) / 256 : 64;
     const dim3 grid(tokens, tiles), carry_grid(segments, tiles);
-    if (out_bf16)
-        stream_conv_kernel<bf16><<<grid, 256, 0, stream>>>(x, weight, state, state_stride, carried_offset, token_segment,
-                                                           seg_q_start, state_slots, static_cast<bf16*>(out), channels, taps);
-    else
-        stream_conv_kernel<float><<<grid, 256, 0, stream>>>(x, weight, state, state_stride, carried_offset, token_segment,
-                                                            seg_q_start, state_slots, static_cast<float*>(out), channels, taps);
+    const bool four = !single_tokens && channels % 4 == 0 && state_stride % 4 == 0 && carried_offset % 4 == 0 &&
+                      reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(state) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(weight) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    if (four) {
+        const dim3 grid4(tokens, (channels / 4 + 255) / 256);
+        if (out_bf16)
+            stream_conv_four_kernel<bf16><<<grid4, 256, 0, stream>>>(x, weight, state, state_stride, carried_offset,
+                                                                     token_segment, seg_q_start, state_slots,
+                                                                     static_cast<bf16*>(out), channels, taps);
+        else
+            stream_conv_four_kernel<float><<<grid4, 256, 0, stream>>>(x, weight, state, state_stride, carried_offset,
+                                                                      token_segment, seg_q_start, state_slots,
+                                                                      static_cast<float*>(out), channels, taps);
+        if (const int err = launch_status()) return err;
+        if (taps == 1) return 0;
+        conv_carry_kernel<float><<<carry_grid, 256, 0, stream>>>(x, channels, state, state_stride, carried_offset, seg_q_start,
+                                                                 seg_q_len, state_slots, channels, taps);
+        return launch_status();
+    }
+#define LAUNCH(T, CARRY)                                                                                              \
+    stream_conv_kernel<T, CARRY><<<grid, 256, 0, stream>>>(x, weight, state, state_stride, carried_offset, token_segment, \
+                                                           seg_q_start, state_slots, static_cast<T*>(out), channels, taps)
+    if (out_bf16) { if (single_tokens) LAUNCH(bf16, true); else LAUNCH(bf16, false); }
+    else { if (single_tokens) LAUNCH(float, true); else LAUNCH(float, false); }
+#undef LAUNCH
     if (const int err = launch_status()) return err;
-    if (taps == 1) return 0;
+    if (taps == 1 || single_tokens) return 0;
     conv_carry_kernel<float><<<carry_grid, 256, 0, stream>>>(x, channels, state, state_stride, carried_offset, seg_q_start,
                                                              seg_q_len, state_slots, channels, taps);
     return launch_status();

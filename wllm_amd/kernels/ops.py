@@ -846,26 +846,31 @@ def causal_conv(inp: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, sta
 
 
 def stream_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, carried_offset: int, token_segment: torch.Tensor,
-                seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor) -> None:
+                seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor,
+                single_tokens: bool = False) -> None:
     """A short causal convolution over time on each channel of the residual stream, added to the stream's own value:
-    out[t, c] = x[t, c] + sum_k weight[c, k] * x[t - (taps - 1) + k, c], the rows before a segment's first token taken
+    out[t, c] = x[t, c] + sum_k weight[k, c] * x[t - (taps - 1) + k, c], the rows before a segment's first token taken
     from the request's carried rows (zeros for a fresh request), which afterwards hold the segment's last taps - 1 rows.
-    x float32 [n, C]; weight float32 [C, taps]; state float32 [slots, W] with the carried rows [taps - 1, C] from column
-    `carried_offset` of row state_slots[segment]; out T [n, C].  float32 sums in the order written."""
+    x float32 [n, C]; weight float32 [taps, C] (a row a tap, the last the current token's); state float32 [slots, W] with the carried rows [taps - 1, C] from column
+    `carried_offset` of row state_slots[segment]; out T [n, C].  float32 sums in the order written.
+    `single_tokens`: the caller knows that every segment is one token (a decode step); the carried rows are then moved
+    by the launch that reads them (the same results, one launch less)."""
     _dense(x, "x", torch.float32)
     _need(x.dim() == 2, "x: expected [n, channels]")
     n, channels = x.shape
     _dense(weight, "weight", torch.float32)
-    _need(weight.dim() == 2 and weight.shape[0] == channels and 1 <= weight.shape[1] <= 64, "weight: expected [channels, taps <= 64]")
-    taps = weight.shape[1]
+    _need(weight.dim() == 2 and weight.shape[1] == channels and 1 <= weight.shape[0] <= 64, "weight: expected [taps <= 64, channels]")
+    taps = weight.shape[0]
     _dense(state, "state", torch.float32)
     _need(state.dim() == 2 and 0 <= carried_offset and carried_offset + (taps - 1) * channels <= state.shape[1],
           "state: a row holds the carried rows from carried_offset")
     _dense(token_segment, "token_segment", torch.int32, (n,))
     _segments(seg_q_start, seg_q_len, state_slots)
     _dense(out, "out", _ACT, (n, channels))
+    _need(not single_tokens or seg_q_start.shape[0] == n, "single_tokens: as many segments as tokens")
     if n:
-        call("stream_conv", x, weight, state, int(carried_offset), token_segment, seg_q_start, seg_q_len, state_slots, out)
+        call("stream_conv", x, weight, state, int(carried_offset), token_segment, seg_q_start, seg_q_len, state_slots, out,
+             **({"single_tokens": True} if single_tokens else {}))
 
 
 def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
@@ -1322,12 +1327,12 @@ def _register_own() -> None:
                     seg_q_start.shape[0], inp.shape[1], weight.shape[1], stream))
     register_op("stream_conv", entry_point="wllm_stream_conv",
                 argtypes=[c_void_p, c_void_p, c_void_p, c_longlong, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                          c_int, c_int, c_int, c_int, c_int, c_void_p],
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
                 launch=lambda fn, stream, x, weight, state, carried_offset, token_segment, seg_q_start, seg_q_len, state_slots,
-                out: fn(
+                out, single_tokens=False: fn(
                     p(x), p(weight), p(state), state.stride(0), carried_offset, p(token_segment), p(seg_q_start), p(seg_q_len),
                     p(state_slots), p(out), int(out.dtype == torch.bfloat16), x.shape[0], seg_q_start.shape[0], x.shape[1],
-                    weight.shape[1], stream))
+                    weight.shape[0], int(single_tokens), stream))
     register_op("ssm_scan", entry_point="wllm_ssm_scan",
                 argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p,
                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],

@@ -275,14 +275,16 @@ class InputConv:
         return {self.spec.weight: ExpectedTensor((self.spec.size, self.spec.taps), role="vector")}
 
     def load(self, fetch) -> None:
-        self.weight = fetch.to_device(fetch.vector(self.spec.weight))      # the taps stay float32
+        # the taps stay float32, a row a tap: the kernel's threads read neighbouring channels of one tap
+        self.weight = fetch.to_device(fetch.vector(self.spec.weight).t().contiguous())
 
     def forward(self, ctx, state: torch.Tensor, offset: int, stream: ResidualStream) -> torch.Tensor:
         n, hidden = stream.x.shape
         stream.settle()         # the convolution reads other tokens' rows of the stream: they take what is pending first
         out = ctx.buffer("conv_in", (n, hidden), ctx.dtype)
+        # (a step of single tokens, a captured graph among them: the carried rows move in the same launch)
         ops.stream_conv(stream.x, self.weight, state, offset, ctx.token_segment, ctx.seg_q_start, ctx.seg_q_len,
-                        ctx.state_slots, out)
+                        ctx.state_slots, out, single_tokens=ctx.max_q_len == 1 and ctx.num_segments == n)
         return out
 
 
