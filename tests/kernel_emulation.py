@@ -242,7 +242,7 @@ class EmulatedKernels:
             v = v - v.mean(-1, keepdim=True)
         return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + recipe.eps) * (recipe.offset + recipe.weight.to(self.acc))
 
-    def norm_add(self, x, delta, delta_norm, out, out_norm, rows):
+    def norm_add(self, x, delta, delta_norm, out, out_norm, rows, conv=None):
         self._count("norm_add")
         idx = rows.long() if rows is not None else slice(None)
         v = x[idx].to(self.acc)
@@ -256,6 +256,16 @@ class EmulatedKernels:
             if rows is None:
                 x.copy_(v)
             v = v.to(self.acc)
+        if conv is not None:
+            weight, state, offset, slots = conv
+            taps, c = weight.shape
+            for r in range(x.shape[0]):
+                carried = state[int(slots[r]), offset:offset + (taps - 1) * c].view(taps - 1, c)
+                seq = torch.cat([carried.to(self.acc), v[r:r + 1]], dim=0)
+                out[r] = (v[r] + (seq * weight.to(self.acc)).sum(0)).to(out.dtype)
+                if taps > 1:
+                    carried.copy_(seq[1:].float())
+            return
         if out is not None:
             out.copy_(self._normed(v, out_norm).to(out.dtype))
 

@@ -116,6 +116,39 @@ def test_the_convolution_of_the_stream_whole_and_in_pieces(dtype, channels, taps
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,taps,stack", [(64, 4, 0), (300, 2, 3), (2048, 3, 0), (48, 1, 2), (600, 9, 0), (4096, 8, 2)])
+def test_settling_the_stream_and_the_convolution_in_one_launch(dtype, hidden, taps, stack):
+    """For a step of single tokens `norm_add` with `conv` gives the bits of `norm_add` and then `stream_conv`, in the
+    stream, in the sublayer's input and in the carried rows."""
+    g = torch.Generator().manual_seed(hidden + taps)
+    n, slots_total, offset = 7, 9, 4
+    x = torch.randn(n, hidden, generator=g)
+    delta = torch.randn(stack, n, hidden, generator=g) if stack else torch.randn(n, hidden, generator=g).to(dtype)
+    norm_w = (1.0 + 0.3 * torch.randn(hidden, generator=g)).to(DEV)
+    w = (torch.randn(taps, hidden, generator=g) * 0.5).to(DEV)
+    state0 = torch.randn(slots_total, offset + (taps - 1) * hidden + 2, generator=g)
+    slots = torch.randperm(slots_total, generator=g)[:n].to(torch.int32).to(DEV)
+    recipe = ops.NormRecipe("layer", norm_w, 1e-5, 0.0)
+    seg = torch.arange(n, dtype=torch.int32, device=DEV)
+    ones = torch.ones(n, dtype=torch.int32, device=DEV)
+    xa, sa = x.clone().to(DEV), state0.clone().to(DEV)
+    out_a = torch.zeros(n, hidden, dtype=dtype, device=DEV)
+    ops.norm_add(xa, delta=delta.to(DEV), delta_norm=recipe)
+    ops.stream_conv(xa, w, sa, offset, seg, seg, ones, slots, out_a, single_tokens=True)
+    xb, sb = x.clone().to(DEV), state0.clone().to(DEV)
+    out_b = torch.zeros(n, hidden, dtype=dtype, device=DEV)
+    ops.norm_add(xb, delta=delta.to(DEV), delta_norm=recipe, out=out_b, conv=(w, sb, offset, slots))
+    assert torch.equal(xa, xb) and torch.equal(out_a, out_b) and torch.equal(sa, sb)
+    d = (delta.sum(0) if stack else delta).double()
+    settled = x.double() + plain.layer_norm(d, norm_w.cpu().double(), 1e-5)
+    close(xb, settled, torch.float32, "the stream", scale=4.0)
+    for r in range(n):
+        carried = state0[int(slots[r]), offset:offset + (taps - 1) * hidden].view(taps - 1, hidden).double()
+        seq = torch.cat([carried, settled[r:r + 1]])
+        close(out_b[r], settled[r] + (seq * w.cpu().double()).sum(0), dtype, f"row {r}", scale=4.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,d,dv", [(2, 16, 32), (3, 10, 12), (1, 130, 5), (4, 64, 72), (1, 256, 40), (5, 4, 130)])
 def test_a_forget_gate_recurrence_whole_and_token_by_token(dtype, heads, d, dv):
     """The recurrence over a prompt, over the same prompt cut into pieces down to single tokens (through state rows

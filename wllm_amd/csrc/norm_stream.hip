@@ -9,7 +9,21 @@
 // for, is the new x under the second norm (the same three kinds; "none" is a cast), in the
 // activation type.  Everything is float32: means, variances as means of squared deviations (two
 // passes over a row held in shared memory), the sum.  One workgroup a row.
+//
+// `conv` (a step in which every row is its request's one new token): out is not a norm of the new x but the new x
+// through a short convolution over time, out[c] = x[c] + sum_k w[k, c] * (the request's k-th carried row, the last tap
+// x itself), and the carried rows (float32 [taps - 1, H] from `carried_offset` of row state_slots[row] of `state`)
+// move up by one and take x: what `stream_conv` does for single tokens, in the launch that settles the stream.
 #include "common.h"
+
+struct NormConv {
+    const float* weight;       // [taps, H], a row a tap; null: no convolution
+    float* state;
+    long long state_stride;
+    long long carried_offset;
+    const int* state_slots;
+    int taps;
+};
 
 constexpr int kNormNone = 0, kNormRms = 1, kNormLayer = 2;
 
@@ -39,12 +53,29 @@ __global__ void __launch_bounds__(1024)
 norm_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, int splits, size_t split_stride, int d_kind,
                 const float* __restrict__ d_weight, float d_eps, float d_offset, const int* __restrict__ rows,
                 TO* __restrict__ out, int o_kind, const float* __restrict__ o_weight, float o_eps, float o_offset,
-                int hidden) {
+                int hidden, NormConv conv) {
     extern __shared__ float row[];
     __shared__ float scratch[16];
     const int orow = blockIdx.x;
     const int irow = rows ? rows[orow] : orow;
     float* xr = x + static_cast<size_t>(irow) * hidden;
+    // The convolution's taps and the carried rows of this thread's (at most two) elements are asked for before anything
+    // else, so that they arrive while the sublayer's product is normalised: a row's time is its chain of trips to memory.
+    constexpr int kHeldTaps = 8;
+    float held_w[2][kHeldTaps], held_c[2][kHeldTaps];
+    const bool held = conv.weight && conv.taps <= kHeldTaps && hidden <= 2 * static_cast<int>(blockDim.x);
+    if (held) {
+        const float* carried = conv.state + static_cast<size_t>(conv.state_slots[orow]) * conv.state_stride + conv.carried_offset;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int i = threadIdx.x + e * blockDim.x;
+#pragma unroll
+            for (int k = 0; k < kHeldTaps; ++k) {
+                held_w[e][k] = (i < hidden && k < conv.taps) ? conv.weight[static_cast<size_t>(k) * hidden + i] : 0.f;
+                held_c[e][k] = (i < hidden && k + 1 < conv.taps) ? carried[static_cast<size_t>(k) * hidden + i] : 0.f;
+            }
+        }
+    }
     if (delta) {
         const TD* dr = delta + static_cast<size_t>(irow) * hidden;
         for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
@@ -67,10 +98,49 @@ norm_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, int splits,
         for (int i = threadIdx.x; i < hidden; i += blockDim.x) row[i] = xr[i];
     }
     if (!out) return;
+    TO* o = out + static_cast<size_t>(orow) * hidden;
+    if (conv.weight) {
+        // (a thread's own elements of the row, and its own columns of the carried rows)
+        float* carried = conv.state + static_cast<size_t>(conv.state_slots[orow]) * conv.state_stride + conv.carried_offset;
+        const int taps = conv.taps;
+        if (held) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int i = threadIdx.x + e * blockDim.x;
+                if (i >= hidden) break;
+                const float now = row[i];
+                float acc = now;
+#pragma unroll
+                for (int k = 0; k < kHeldTaps; ++k) {
+                    if (k + 1 < taps) {
+                        acc = fmaf(held_w[e][k], held_c[e][k], acc);
+                        if (k > 0) carried[static_cast<size_t>(k - 1) * hidden + i] = held_c[e][k];
+                    } else if (k + 1 == taps) {
+                        acc = fmaf(held_w[e][k], now, acc);
+                    }
+                }
+                if (taps > 1) carried[static_cast<size_t>(taps - 2) * hidden + i] = now;
+                o[i] = from_float<TO>(acc);
+            }
+            return;
+        }
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+            const float now = row[i];
+            float acc = now;
+            for (int k = 0; k + 1 < taps; ++k) {
+                const float v = carried[static_cast<size_t>(k) * hidden + i];
+                acc = fmaf(conv.weight[static_cast<size_t>(k) * hidden + i], v, acc);
+                if (k > 0) carried[static_cast<size_t>(k - 1) * hidden + i] = v;
+            }
+            acc = fmaf(conv.weight[static_cast<size_t>(taps - 1) * hidden + i], now, acc);
+            if (taps > 1) carried[static_cast<size_t>(taps - 2) * hidden + i] = now;
+            o[i] = from_float<TO>(acc);
+        }
+        return;
+    }
     __syncthreads();
     float mean, inv;
     row_stats(row, hidden, o_kind, o_eps, scratch, mean, inv);
-    TO* o = out + static_cast<size_t>(orow) * hidden;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = row[i];
         if (o_kind != kNormNone) v = (v - mean) * inv * (o_offset + o_weight[i]);
@@ -82,8 +152,12 @@ norm_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, int splits,
 WLLM_API int wllm_norm_add(float* x, const void* delta, int delta_type, int splits, long long split_stride, int d_kind,
                            const float* d_weight, float d_eps, float d_offset, const int* rows, void* out, int out_type,
                            int o_kind, const float* o_weight, float o_eps, float o_offset, int num_rows, int hidden,
-                           hipStream_t stream) {
+                           const float* conv_weight, int conv_taps, float* conv_state, long long conv_state_stride,
+                           long long conv_carried_offset, const int* conv_state_slots, hipStream_t stream) {
     if (num_rows <= 0) return 0;
+    if (conv_weight && (!out || rows || o_kind != kNormNone || conv_taps < 1 || conv_taps > 64 || !conv_state || !conv_state_slots))
+        return -1;
+    const NormConv conv{conv_weight, conv_state, conv_state_stride, conv_carried_offset, conv_state_slots, conv_taps};
     if (hidden <= 0 || hidden > 16384 || !x) return -1;
     if (d_kind < 0 || d_kind > 2 || o_kind < 0 || o_kind > 2) return -1;
     if (delta && d_kind != kNormNone && !d_weight) return -1;
@@ -101,7 +175,7 @@ WLLM_API int wllm_norm_add(float* x, const void* delta, int delta_type, int spli
     norm_add_kernel<TD, TO><<<num_rows, threads, smem, stream>>>(x, static_cast<const TD*>(delta), splits,            \
                                                               static_cast<size_t>(split_stride), d_kind, d_weight,   \
                                                               d_eps, d_offset, rows, static_cast<TO*>(out), o_kind,   \
-                                                              o_weight, o_eps, o_offset, hidden)
+                                                              o_weight, o_eps, o_offset, hidden, conv)
     if (delta_type && out_type) LAUNCH(bf16, bf16);
     else if (delta_type) LAUNCH(bf16, float);
     else if (out_type) LAUNCH(float, bf16);

@@ -725,14 +725,17 @@ class NormRecipe:
 
 def norm_add(x: torch.Tensor, *, delta: Optional[torch.Tensor] = None, delta_norm: Optional[NormRecipe] = None,
              out: Optional[torch.Tensor] = None, out_norm: Optional[NormRecipe] = None,
-             rows: Optional[torch.Tensor] = None) -> None:
+             rows: Optional[torch.Tensor] = None, conv: Optional[tuple] = None) -> None:
     """x += delta_norm(delta); out = out_norm(x), all in float32.
 
     x float32 [n, H], the residual stream.  delta T [n, H] or a stack float32 [S, n, H] of partial sums
     added in order; with `delta_norm` it is normalised before it is added (a norm behind a sublayer).
     out T or float32 [m, H] (optional): the new x under `out_norm` (None: as it is, cast).  Without
     `rows`, m = n and the sum is written back to x.  With `rows` (int32 [m]) only those rows are read,
-    x is left alone and out[i] belongs to row rows[i]."""
+    x is left alone and out[i] belongs to row rows[i].
+    `conv` = (weight, state, carried_offset, state_slots), for a step in which every row is its request's one new
+    token: out is then the new x through `stream_conv` with `single_tokens` (weight float32 [taps, H]; the carried rows
+    of row i lie in row state_slots[i] of state), in the same launch; neither `out_norm` nor `rows` goes with it."""
     _dense(x, "x", torch.float32)
     _need(x.dim() == 2, "x: expected [tokens, hidden]")
     n, h = x.shape
@@ -758,8 +761,19 @@ def norm_add(x: torch.Tensor, *, delta: Optional[torch.Tensor] = None, delta_nor
         _dense(out, "out", _ACT, (m, h))
     else:
         _need(out_norm is None, "out_norm without out")
+    extra = {}
+    if conv is not None:
+        weight, state, carried_offset, state_slots = conv
+        _need(out is not None and out_norm is None and rows is None, "conv: with out, without out_norm and rows")
+        _dense(weight, "conv weight", torch.float32)
+        _need(weight.dim() == 2 and weight.shape[1] == h and 1 <= weight.shape[0] <= 64, "conv weight: expected [taps <= 64, hidden]")
+        _dense(state, "conv state", torch.float32)
+        _need(state.dim() == 2 and 0 <= carried_offset and carried_offset + (weight.shape[0] - 1) * h <= state.shape[1],
+              "conv state: a row holds the carried rows from carried_offset")
+        _dense(state_slots, "conv state_slots", torch.int32, (n,))
+        extra["conv"] = (weight, state, int(carried_offset), state_slots)
     if m and (delta is not None or out is not None):
-        call("norm_add", x, delta, delta_norm, out, out_norm, rows)
+        call("norm_add", x, delta, delta_norm, out, out_norm, rows, **extra)
 
 
 def band_norm(bands: list, eps: float) -> None:
@@ -1277,7 +1291,7 @@ def _register_own() -> None:
                 launch=add)
 
 
-    def norm_add_launch(fn, stream, x, delta, delta_norm, out, out_norm, rows):
+    def norm_add_launch(fn, stream, x, delta, delta_norm, out, out_norm, rows, conv=None):
         splits, stride = 1, 0
         if delta is not None and delta.dim() == 3:
             splits, stride = delta.shape[0], delta.shape[1] * delta.shape[2]
@@ -1287,11 +1301,14 @@ def _register_own() -> None:
 
         return fn(p(x), p(delta), int(delta is not None and delta.dtype == torch.bfloat16), splits, stride,
                   *recipe(delta_norm), p(rows), p(out), int(out is not None and out.dtype == torch.bfloat16),
-                  *recipe(out_norm), out.shape[0] if out is not None else x.shape[0], x.shape[1], stream)
+                  *recipe(out_norm), out.shape[0] if out is not None else x.shape[0], x.shape[1],
+                  *((p(conv[0]), conv[0].shape[0], p(conv[1]), conv[1].stride(0), conv[2], p(conv[3])) if conv is not None
+                    else (p(None), 0, p(None), 0, 0, p(None))), stream)
 
     register_op("norm_add", entry_point="wllm_norm_add",
                 argtypes=[c_void_p, c_void_p, c_int, c_int, c_longlong, c_int, c_void_p, c_float, c_float, c_void_p, c_void_p,
-                          c_int, c_int, c_void_p, c_float, c_float, c_int, c_int, c_void_p],
+                          c_int, c_int, c_void_p, c_float, c_float, c_int, c_int, c_void_p, c_int, c_void_p, c_longlong,
+                          c_longlong, c_void_p, c_void_p],
                 launch=norm_add_launch)
 
     def band_norm_launch(fn, stream, bands, eps):

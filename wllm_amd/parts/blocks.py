@@ -280,11 +280,18 @@ class InputConv:
 
     def forward(self, ctx, state: torch.Tensor, offset: int, stream: ResidualStream) -> torch.Tensor:
         n, hidden = stream.x.shape
-        stream.settle()         # the convolution reads other tokens' rows of the stream: they take what is pending first
         out = ctx.buffer("conv_in", (n, hidden), ctx.dtype)
-        # (a step of single tokens, a captured graph among them: the carried rows move in the same launch)
+        single = ctx.max_q_len == 1 and ctx.num_segments == n       # a step of single tokens, a captured graph among them
+        if single and stream.pending is not None and stream.pending_bias is None:
+            # no token reads another's row: the launch that settles the stream also convolves and moves the carried rows
+            ops.norm_add(stream.x, delta=stream.pending, delta_norm=stream.pending_norm, out=out,
+                         conv=(self.weight, state, offset, ctx.state_slots))
+            stream.pending = stream.pending_norm = None
+            stream.sumsq = None
+            return out
+        stream.settle()         # the convolution reads other tokens' rows of the stream: they take what is pending first
         ops.stream_conv(stream.x, self.weight, state, offset, ctx.token_segment, ctx.seg_q_start, ctx.seg_q_len,
-                        ctx.state_slots, out, single_tokens=ctx.max_q_len == 1 and ctx.num_segments == n)
+                        ctx.state_slots, out, single_tokens=single)
         return out
 
 
